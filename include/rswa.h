@@ -1,0 +1,172 @@
+/*
+ * rswa.h — C ABI of the MI355X (gfx950) kernels behind ring_swa's single-GPU
+ * attention path.
+ *
+ * Plain C: raw device pointers, element strides, sizes.  No torch types.  Every
+ * call only enqueues work on `stream` (a hipStream_t passed as void*); nothing
+ * synchronises the device and nothing allocates or frees device memory — the
+ * caller owns all buffers, scratch included.  Functions return 0 on success and
+ * a negative rswa_status otherwise; rswa_last_error() gives the message of the
+ * calling thread's last failure.
+ *
+ * Each entry point replaces one interface of the upstream Python package
+ * (paths relative to its repository root):
+ *
+ *   rswa_merge_attn_out   ring_swa/ops/merge.py:150-193  (triton_merge_attn_out;
+ *                         torch twin :16-50; selector :196-208)
+ *   rswa_attn_fwd         ring_swa/ops/wrap_flash.py:168-200 (wrapped_flash_attn_fwd)
+ *                         and :203-273 (wrapped_flash_attn_fwd_varlen); also the
+ *                         forward half of flash_attn_func / flash_attn_varlen_func at
+ *                         ring_swa/sliding_window/nonvarlen.py:379-386 and
+ *                         ring_swa/sliding_window/varlen.py:406-417
+ *   rswa_attn_bwd         ring_swa/ops/wrap_flash.py:276-327 (wrapped_flash_attn_bwd)
+ *                         and :330-429 (wrapped_flash_attn_bwd_varlen)
+ *   rswa_attn_bwd_workspace_bytes   (sizing helper for the scratch rswa_attn_bwd
+ *                         needs; upstream flash-attn allocates the same internally)
+ */
+#ifndef RSWA_H
+#define RSWA_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RSWA_VERSION 1
+
+typedef enum rswa_status {
+  RSWA_OK = 0,
+  RSWA_ERR_INVALID = -1,     /* bad argument / inconsistent shapes            */
+  RSWA_ERR_UNSUPPORTED = -2, /* dtype / head_dim / stride the kernels lack    */
+  RSWA_ERR_LAUNCH = -3       /* HIP reported an error at launch               */
+} rswa_status;
+
+typedef enum rswa_dtype {
+  RSWA_BF16 = 0,
+  RSWA_F16 = 1,
+  RSWA_F32 = 2,
+  RSWA_F64 = 3
+} rswa_dtype;
+
+/*
+ * In-place log-sum-exp merge of a new partial into a running one:
+ *   w_old = sigmoid(lse - lse_new), w_new = sigmoid(lse_new - lse)
+ *   o   <- w_old * o + w_new * o_new
+ *   lse <- max(lse, lse_new) + log1p(exp(-|lse_new - lse|))
+ * lse = -inf is the identity element on either side; both -inf gives
+ * (o = 0, lse = -inf).  Arithmetic is fp32 whatever the storage types
+ * (ring_swa/ops/merge.py:134-135 down-casts fp64 LSE the same way).
+ *
+ * o, o_new: logical [batch, seqlen, heads, head_dim]; lse, lse_new: logical
+ * [batch, heads, seqlen].  Strides are in ELEMENTS, arrays of 4 (b,s,h,d) and
+ * 3 (b,h,s); the head_dim stride must be 1.  Sliced / expanded views are fine.
+ * o_dtype, o_new_dtype in {BF16, F16, F32}; lse_dtype, lse_new_dtype in
+ * {F32, F64}.  head_dim must be a multiple of 8, at most 256.
+ */
+int rswa_merge_attn_out(void* o, int o_dtype, const int64_t* o_stride,
+                        void* lse, int lse_dtype, const int64_t* lse_stride,
+                        const void* o_new, int o_new_dtype, const int64_t* o_new_stride,
+                        const void* lse_new, int lse_new_dtype, const int64_t* lse_new_stride,
+                        int64_t batch, int64_t seqlen, int64_t heads, int64_t head_dim,
+                        void* stream);
+
+/*
+ * One attention block, forward or backward.
+ *
+ * Dense mode (cu_seqlens_q == NULL): q/out/dout/dq are [batch, seqlen_q,
+ * heads_q, head_dim], k/v/dk/dv are [batch, seqlen_k, heads_kv, head_dim], lse
+ * is fp32 [batch, heads_q, seqlen_q].
+ * Packed mode (cu_seqlens_q and cu_seqlens_k given, int32 device arrays of
+ * batch + 1 entries): tensors are [total, heads, head_dim], lse is fp32
+ * [heads_q, total_q]; the batch strides are ignored; seqlen_q / seqlen_k are
+ * upper bounds on the per-sequence lengths (they only size the launch) and
+ * total_q / total_k are the packed row counts.
+ *
+ * Strides are in elements: *_stride[0] batch, [1] row (token), [2] head; the
+ * head_dim stride must be 1 and every row must start 16-byte aligned.
+ * lse_stride: [0] batch, [1] head, [2] row.
+ *
+ * Mask (flash-attn's local-window rule, bottom-right aligned): with
+ * shift = len_k - len_q of the sequence, key j is visible from query i iff
+ *   i + shift - window_left <= j <= i + shift + window_right
+ * where a negative window bound means unbounded and causal != 0 forces
+ * window_right = 0.  num_sink > 0 additionally makes keys j < num_sink visible
+ * whenever they satisfy the right bound (attention sinks at the sequence head).
+ * Rows with no visible key produce out = 0, lse = -inf.
+ *
+ * lse is the natural-log sum of exp(softmax_scale * q.k) over visible keys.
+ *
+ * Backward takes the caller's out / lse — they may be the result of merging
+ * several blocks, which is how the ring's "merge backward" is realised
+ * (ring_swa/sliding_window/nonvarlen.py:242-253) — and OVERWRITES dq, dk, dv
+ * (rows/keys that receive nothing are written as zero).  dk/dv are reduced over
+ * the heads_q / heads_kv query heads that share a kv head.  dq is accumulated
+ * with fp32 atomics in `workspace`, so its low-order bits are not run-to-run
+ * deterministic (upstream flash-attn runs with deterministic=False as well,
+ * ring_swa/ops/wrap_flash.py:61).
+ */
+typedef struct rswa_attn_params {
+  int32_t dtype;    /* RSWA_BF16 or RSWA_F16: type of q,k,v,out,dout,dq,dk,dv */
+  int32_t head_dim; /* 64 or 128                                             */
+  int32_t batch;
+  int32_t heads_q;
+  int32_t heads_kv;
+  int32_t seqlen_q; /* dense: exact; packed: upper bound of per-sequence len  */
+  int32_t seqlen_k;
+  int64_t total_q;  /* packed mode only                                       */
+  int64_t total_k;
+  const int32_t* cu_seqlens_q; /* NULL => dense                               */
+  const int32_t* cu_seqlens_k;
+
+  float softmax_scale;
+  int32_t window_left;  /* < 0: unbounded */
+  int32_t window_right; /* < 0: unbounded */
+  int32_t causal;
+  int32_t num_sink;
+
+  const void* q;
+  const void* k;
+  const void* v;
+  int64_t q_stride[3];
+  int64_t k_stride[3];
+  int64_t v_stride[3];
+
+  void* out;  /* fwd: written.  bwd: read (const) */
+  int64_t out_stride[3];
+  float* lse; /* fwd: written.  bwd: read (const) */
+  int64_t lse_stride[3];
+
+  /* backward only */
+  const void* dout;
+  int64_t dout_stride[3];
+  void* dq;
+  void* dk;
+  void* dv;
+  int64_t dq_stride[3];
+  int64_t dk_stride[3];
+  int64_t dv_stride[3];
+  void* workspace;        /* >= rswa_attn_bwd_workspace_bytes(), 256-byte aligned */
+  uint64_t workspace_bytes;
+} rswa_attn_params;
+
+int rswa_attn_fwd(const rswa_attn_params* p, void* stream);
+int rswa_attn_bwd(const rswa_attn_params* p, void* stream);
+
+/* Scratch rswa_attn_bwd needs for these shapes (fp32 dq accumulator + row sums). */
+uint64_t rswa_attn_bwd_workspace_bytes(const rswa_attn_params* p);
+
+/* Message of the calling thread's last failed call ("" if none). */
+const char* rswa_last_error(void);
+
+/* RSWA_VERSION the library was built from. */
+int rswa_version(void);
+
+/* sizeof(rswa_attn_params) the library was built with (binding self-check). */
+uint64_t rswa_sizeof_attn_params(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RSWA_H */

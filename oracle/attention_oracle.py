@@ -258,15 +258,15 @@ def merge(o, lse, o_new, lse_new):
     ``o [B,S,H,D]``, ``lse [B,H,S]``.  Returns ``(o_merged, lse_merged)`` in the
     dtype of ``o`` / ``lse``; arithmetic in fp32 as the Triton kernel does
     (``:134-135``) unless ``lse`` is fp64 *and* ``o`` is fp64.  ``-inf`` on either
-    side is the identity; both ``-inf`` stays ``(0-weighted, -inf)``.
+    side is the identity; both ``-inf`` gives ``(0, -inf)`` (the reference yields NaN there).
     """
     cd = torch.float64 if (lse.dtype == torch.float64 and o.dtype == torch.float64) else torch.float32
     a = lse.to(cd)
     b = lse_new.to(cd)
     both_empty = torch.isinf(a) & torch.isinf(b) & (a < 0) & (b < 0)
     diff = torch.where(both_empty, torch.zeros_like(a), b - a)
-    w_old = torch.sigmoid(-diff)
-    w_new = torch.sigmoid(diff)
+    w_old = torch.sigmoid(-diff).masked_fill(both_empty, 0.0)
+    w_new = torch.sigmoid(diff).masked_fill(both_empty, 0.0)
     w_old_b = w_old.movedim(1, 2).unsqueeze(-1)
     w_new_b = w_new.movedim(1, 2).unsqueeze(-1)
     o_m = o.to(cd) * w_old_b + o_new.to(cd) * w_new_b

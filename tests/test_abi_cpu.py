@@ -1,0 +1,84 @@
+"""CPU-side checks of the C-ABI boundary: the library loads, exports every
+symbol the header declares, the Python struct mirrors the C struct, and
+argument validation fails cleanly without touching a GPU."""
+import ctypes
+import importlib.util
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PKG = os.path.join(ROOT, "ring-sliding-window-attention_amd")
+HEADER = os.path.join(ROOT, "include", "rswa.h")
+
+
+def _ensure_built():
+    lib = os.path.join(PKG, "lib", "librswa.so")
+    if not os.path.exists(lib):
+        spec = importlib.util.spec_from_file_location("rswa_build", os.path.join(PKG, "build.py"))
+        mod = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(mod)
+        mod.build()
+    return lib
+
+
+def _declared_symbols():
+    src = open(HEADER).read()
+    src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
+    return sorted(set(re.findall(r"\b(rswa_[a-z_0-9]+)\s*\(", src)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ctypes.CDLL(_ensure_built())
+    names = _declared_symbols()
+    assert {"rswa_merge_attn_out", "rswa_attn_fwd", "rswa_attn_bwd", "rswa_last_error",
+            "rswa_attn_bwd_workspace_bytes"} <= set(names)
+    for n in names:
+        assert hasattr(lib, n), f"librswa.so does not export {n}"
+
+
+def test_python_struct_matches_c_struct():
+    _ensure_built()
+    from ring_swa import _lib
+
+    L = _lib.lib()
+    assert L.rswa_sizeof_attn_params() == ctypes.sizeof(_lib.AttnParams)
+    assert L.rswa_version() == 1
+
+
+def test_header_cites_reference_interfaces():
+    src = open(HEADER).read()
+    for cite in ("ring_swa/ops/merge.py:150", "ring_swa/ops/wrap_flash.py:168",
+                 "ring_swa/ops/wrap_flash.py:276"):
+        assert cite in src
+
+
+def test_merge_argument_validation_needs_no_gpu():
+    _ensure_built()
+    from ring_swa import _lib
+
+    L = _lib.lib()
+    st4 = _lib.i64x4((8 * 4 * 128, 4 * 128, 128, 1))
+    st3 = _lib.i64x3((4 * 8, 8, 1))
+    # head_dim not a multiple of 8 -> unsupported, reported through rswa_last_error
+    rc = L.rswa_merge_attn_out(16, 2, st4, 16, 2, st3, 16, 0, st4, 16, 2, st3, 1, 8, 4, 100, None)
+    assert rc == -2 and b"head_dim" in L.rswa_last_error()
+    # null tensor -> invalid
+    rc = L.rswa_merge_attn_out(None, 2, st4, 16, 2, st3, 16, 0, st4, 16, 2, st3, 1, 8, 4, 128, None)
+    assert rc == -1
+    # empty problem is a no-op
+    rc = L.rswa_merge_attn_out(None, 2, st4, None, 2, st3, None, 0, st4, None, 2, st3, 0, 8, 4, 128,
+                               None)
+    assert rc == 0
+
+
+def test_ops_refuse_cpu_tensors():
+    _ensure_built()
+    from ring_swa.ops import merge_attn_out
+
+    o = torch.zeros(1, 8, 2, 128)
+    l = torch.zeros(1, 2, 8)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        merge_attn_out(o, l, o.clone(), l.clone())
