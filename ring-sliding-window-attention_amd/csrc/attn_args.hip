@@ -1,0 +1,126 @@
+// Host-side validation of rswa_attn_params and translation to kernel arguments.
+#include "attn_common.h"
+
+namespace rswa {
+
+static uint64_t align_up(uint64_t x, uint64_t a) { return (x + a - 1) / a * a; }
+
+static uint64_t dq_acc_bytes(const rswa_attn_params* p) {
+  const uint64_t rows = p->cu_seqlens_q ? (uint64_t)p->total_q
+                                        : (uint64_t)p->batch * (uint64_t)p->seqlen_q;
+  return align_up(rows * (uint64_t)p->heads_q * (uint64_t)p->head_dim * sizeof(float), 256);
+}
+
+static uint64_t delta_bytes(const rswa_attn_params* p) {
+  const uint64_t rows = p->cu_seqlens_q ? (uint64_t)p->total_q
+                                        : (uint64_t)p->batch * (uint64_t)p->seqlen_q;
+  return align_up(rows * (uint64_t)p->heads_q * sizeof(float), 256);
+}
+
+uint64_t bwd_workspace_bytes(const rswa_attn_params* p) {
+  if (!p || p->batch <= 0 || p->heads_q <= 0 || p->head_dim <= 0) return 0;
+  return dq_acc_bytes(p) + delta_bytes(p);
+}
+
+static bool rows_aligned(const void* ptr, const int64_t* st) {
+  if (((uintptr_t)ptr) % 16) return false;
+  for (int i = 0; i < 3; i++)
+    if (st[i] % 8) return false;
+  return true;
+}
+
+int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a) {
+  RSWA_REQUIRE(p != nullptr, RSWA_ERR_INVALID, "attn: null params");
+  RSWA_REQUIRE(p->dtype == RSWA_BF16 || p->dtype == RSWA_F16, RSWA_ERR_UNSUPPORTED,
+               "attn: dtype %d (only bf16 and fp16)", p->dtype);
+  RSWA_REQUIRE(p->head_dim == 64 || p->head_dim == 128, RSWA_ERR_UNSUPPORTED,
+               "attn: head_dim %d (only 64 and 128)", p->head_dim);
+  RSWA_REQUIRE(p->batch > 0 && p->heads_q > 0 && p->heads_kv > 0, RSWA_ERR_INVALID,
+               "attn: batch/heads must be positive");
+  RSWA_REQUIRE(p->heads_q % p->heads_kv == 0, RSWA_ERR_INVALID,
+               "attn: heads_q %d not a multiple of heads_kv %d", p->heads_q, p->heads_kv);
+  RSWA_REQUIRE(p->seqlen_q >= 0 && p->seqlen_k >= 0, RSWA_ERR_INVALID, "attn: negative seqlen");
+  RSWA_REQUIRE(p->softmax_scale > 0.f && p->softmax_scale < 1e30f, RSWA_ERR_INVALID,
+               "attn: softmax_scale must be positive and finite");
+  RSWA_REQUIRE(p->num_sink >= 0, RSWA_ERR_INVALID, "attn: negative num_sink");
+  const bool packed = p->cu_seqlens_q != nullptr || p->cu_seqlens_k != nullptr;
+  if (packed) {
+    RSWA_REQUIRE(p->cu_seqlens_q && p->cu_seqlens_k, RSWA_ERR_INVALID,
+                 "attn: packed mode needs both cu_seqlens_q and cu_seqlens_k");
+    RSWA_REQUIRE(p->total_q >= 0 && p->total_k >= 0, RSWA_ERR_INVALID, "attn: negative totals");
+    RSWA_REQUIRE(p->total_q < (1ll << 31) && p->total_k < (1ll << 31), RSWA_ERR_INVALID,
+                 "attn: totals out of range");
+  }
+  RSWA_REQUIRE(p->q && p->k && p->v && p->out && p->lse, RSWA_ERR_INVALID, "attn: null tensor");
+  RSWA_REQUIRE(rows_aligned(p->q, p->q_stride) && rows_aligned(p->k, p->k_stride) &&
+                   rows_aligned(p->v, p->v_stride) && rows_aligned(p->out, p->out_stride),
+               RSWA_ERR_UNSUPPORTED, "attn: q/k/v/out rows must start 16-byte aligned");
+  RSWA_REQUIRE(((uintptr_t)p->lse) % 4 == 0, RSWA_ERR_UNSUPPORTED, "attn: lse misaligned");
+
+  a.q = p->q;
+  a.k = p->k;
+  a.v = p->v;
+  a.out = p->out;
+  a.lse = p->lse;
+  a.dout = p->dout;
+  a.dq = p->dq;
+  a.dk = p->dk;
+  a.dv = p->dv;
+  a.dq_acc = nullptr;
+  a.delta = nullptr;
+  a.cu_q = p->cu_seqlens_q;
+  a.cu_k = p->cu_seqlens_k;
+  for (int i = 0; i < 3; i++) {
+    a.q_st[i] = p->q_stride[i];
+    a.k_st[i] = p->k_stride[i];
+    a.v_st[i] = p->v_stride[i];
+    a.o_st[i] = p->out_stride[i];
+    a.lse_st[i] = p->lse_stride[i];
+    a.do_st[i] = p->dout_stride[i];
+    a.dq_st[i] = p->dq_stride[i];
+    a.dk_st[i] = p->dk_stride[i];
+    a.dv_st[i] = p->dv_stride[i];
+  }
+  if (packed) {
+    a.q_st[0] = a.k_st[0] = a.v_st[0] = a.o_st[0] = a.lse_st[0] = 0;
+    a.do_st[0] = a.dq_st[0] = a.dk_st[0] = a.dv_st[0] = 0;
+  }
+  a.rows_q = packed ? p->total_q : (int64_t)p->batch * p->seqlen_q;
+  a.batch = p->batch;
+  a.heads_q = p->heads_q;
+  a.heads_kv = p->heads_kv;
+  a.group = p->heads_q / p->heads_kv;
+  a.seqlen_q = p->seqlen_q;
+  a.seqlen_k = p->seqlen_k;
+  a.wl = p->window_left < 0 ? -1 : p->window_left;
+  a.wr = p->causal ? 0 : (p->window_right < 0 ? -1 : p->window_right);
+  a.n_sink = p->num_sink;
+  a.n_tile = 0;
+  a.n_work = 0;
+  a.scale = p->softmax_scale;
+  a.scale_log2 = p->softmax_scale * kLog2e;
+
+  if (backward) {
+    RSWA_REQUIRE(p->dout && p->dq && p->dk && p->dv, RSWA_ERR_INVALID, "attn_bwd: null tensor");
+    RSWA_REQUIRE(rows_aligned(p->dout, p->dout_stride) && rows_aligned(p->dq, p->dq_stride) &&
+                     rows_aligned(p->dk, p->dk_stride) && rows_aligned(p->dv, p->dv_stride),
+                 RSWA_ERR_UNSUPPORTED, "attn_bwd: dout/dq/dk/dv rows must start 16-byte aligned");
+    const uint64_t need = bwd_workspace_bytes(p);
+    RSWA_REQUIRE(p->workspace != nullptr || need == 0, RSWA_ERR_INVALID,
+                 "attn_bwd: null workspace");
+    RSWA_REQUIRE(p->workspace_bytes >= need, RSWA_ERR_INVALID,
+                 "attn_bwd: workspace %llu bytes < required %llu",
+                 (unsigned long long)p->workspace_bytes, (unsigned long long)need);
+    RSWA_REQUIRE(((uintptr_t)p->workspace) % 256 == 0, RSWA_ERR_INVALID,
+                 "attn_bwd: workspace must be 256-byte aligned");
+    a.dq_acc = (float*)p->workspace;
+    a.delta = (float*)((char*)p->workspace + dq_acc_bytes(p));
+  }
+  return RSWA_OK;
+}
+
+}  // namespace rswa
+
+extern "C" uint64_t rswa_attn_bwd_workspace_bytes(const rswa_attn_params* p) {
+  return rswa::bwd_workspace_bytes(p);
+}

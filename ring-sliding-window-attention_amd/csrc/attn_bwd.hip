@@ -1,5 +1,4 @@
-#include "rswa_common.h"
+#include "attn_common.h"
 extern "C" int rswa_attn_bwd(const rswa_attn_params* p, void* stream) {
   return rswa::fail(RSWA_ERR_UNSUPPORTED, "attn_bwd: not built yet");
 }
-extern "C" uint64_t rswa_attn_bwd_workspace_bytes(const rswa_attn_params* p) { return 0; }

@@ -1,0 +1,156 @@
+// Device-side helpers shared by the attention forward and backward kernels.
+//
+// Register layouts used throughout (wave64, gfx950), verified on hardware:
+//   v_mfma_f32_32x32x16 A (32 x 16): lane l holds row l%32, k = 8*(l/32) .. +7
+//                       B (16 x 32): lane l holds col l%32, k = 8*(l/32) .. +7
+//                       C (32 x 32): lane l holds col l%32, reg i is row
+//                                    8*(i/4) + 4*(l/32) + i%4
+//   ds_read_b64_tr_b16: within each group of 16 lanes, lane i supplies the
+//                       address of 4 consecutive 16-bit elements; it receives
+//                       element i%4 of lanes (i/4), 4+(i/4), 8+(i/4), 12+(i/4),
+//                       i.e. column i of the 4 x 16 block whose row r is the
+//                       concatenation of lanes 4r .. 4r+3.
+#pragma once
+
+#include "rswa_common.h"
+
+namespace rswa {
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+// Kernel-side view of rswa_attn_params (strides in elements).
+struct AttnArgs {
+  const void* q;
+  const void* k;
+  const void* v;
+  void* out;
+  float* lse;
+  const void* dout;
+  void* dq;
+  void* dk;
+  void* dv;
+  float* dq_acc;  // fp32 [rows_q, heads_q, head_dim] packed, inside the workspace
+  float* delta;   // fp32 [heads_q, rows_q] packed, inside the workspace
+  const int32_t* cu_q;
+  const int32_t* cu_k;
+  int64_t q_st[3], k_st[3], v_st[3], o_st[3], do_st[3], dq_st[3], dk_st[3], dv_st[3], lse_st[3];
+  int64_t rows_q;  // batch * seqlen_q (dense) or total_q (packed)
+  int32_t batch, heads_q, heads_kv, group;  // group = heads_q / heads_kv
+  int32_t seqlen_q, seqlen_k;
+  int32_t wl, wr, n_sink;  // wl/wr < 0: unbounded
+  int32_t n_tile;          // tiles per sequence (dense) / total tile slots (packed)
+  int32_t n_work;          // logical blocks
+  float scale, scale_log2;
+};
+
+struct SeqInfo {
+  int64_t q_row0, k_row0;  // first row of the sequence in the (batch-strided or packed) tensor
+  int64_t q_base, k_base;  // element offset of the batch (dense) — 0 in packed mode
+  int32_t len_q, len_k;
+  int32_t batch_idx;
+};
+
+// XCD-aware block id: consecutive logical ids land on the same XCD (8 XCDs,
+// hardware deals physical block ids round-robin), so that blocks sharing K/V
+// tiles share an L2.  The grid is padded to a multiple of 8; returns -1 for pad.
+__device__ __forceinline__ int logical_block_id(int n_work) {
+  const int per_xcd = (int)gridDim.x >> 3;
+  const int id = ((int)blockIdx.x & 7) * per_xcd + ((int)blockIdx.x >> 3);
+  return id < n_work ? id : -1;
+}
+
+static inline unsigned padded_grid(int64_t n_work) { return (unsigned)(ceil_div(n_work, 8) * 8); }
+
+// Mask bounds of one query row i (local index): visible keys are
+//   j <= hi  and  (j >= lo or j < n_sink);   hi already clipped to len_k - 1.
+struct RowBounds {
+  int lo, hi;
+};
+
+__device__ __forceinline__ RowBounds row_bounds(const AttnArgs& a, int i, int len_q, int len_k) {
+  RowBounds r;
+  const int shift = len_k - len_q;
+  r.hi = (a.wr >= 0) ? min(len_k - 1, i + shift + a.wr) : len_k - 1;
+  r.lo = (a.wl >= 0) ? max(0, i + shift - a.wl) : 0;
+  if (i >= len_q) r.hi = -1;  // rows past the end see nothing
+  return r;
+}
+
+// Locate tile `t` (counted along the sequence axis `which`: 0 = q, 1 = k) of
+// granularity `tile` in packed mode.  Returns false if t is past the last tile.
+__device__ __forceinline__ bool locate_packed(const AttnArgs& a, int t, int tile, bool along_k,
+                                              SeqInfo& s, int& tile_in_seq) {
+  const int32_t* cu = along_k ? a.cu_k : a.cu_q;
+  int acc = 0;
+  for (int b = 0; b < a.batch; b++) {
+    const int len = cu[b + 1] - cu[b];
+    const int nt = (len + tile - 1) / tile;
+    if (t < acc + nt) {
+      s.batch_idx = b;
+      s.q_row0 = a.cu_q[b];
+      s.k_row0 = a.cu_k[b];
+      s.len_q = a.cu_q[b + 1] - a.cu_q[b];
+      s.len_k = a.cu_k[b + 1] - a.cu_k[b];
+      s.q_base = 0;
+      s.k_base = 0;
+      tile_in_seq = t - acc;
+      return true;
+    }
+    acc += nt;
+  }
+  return false;
+}
+
+template <typename T>
+struct Mma;
+
+template <>
+struct Mma<__bf16> {
+  using V8 = bf16x8;
+  using V4 = bf16x4;
+  static __device__ __forceinline__ f32x16 mfma32(V8 a, V8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ V8 pack(const float* x) {
+    f32x8 f = {x[0], x[1], x[2], x[3], x[4], x[5], x[6], x[7]};
+    return __builtin_convertvector(f, V8);
+  }
+  static __device__ __forceinline__ V4 pack4(float a, float b, float c, float d) {
+    f32x4 f = {a, b, c, d};
+    return __builtin_convertvector(f, V4);
+  }
+};
+
+template <>
+struct Mma<_Float16> {
+  using V8 = f16x8;
+  using V4 = f16x4;
+  static __device__ __forceinline__ f32x16 mfma32(V8 a, V8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ V8 pack(const float* x) {
+    f32x8 f = {x[0], x[1], x[2], x[3], x[4], x[5], x[6], x[7]};
+    return __builtin_convertvector(f, V8);
+  }
+  static __device__ __forceinline__ V4 pack4(float a, float b, float c, float d) {
+    f32x4 f = {a, b, c, d};
+    return __builtin_convertvector(f, V4);
+  }
+};
+
+typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+
+// max / sum across the two half-waves (lane l <-> lane l ^ 32).
+__device__ __forceinline__ float halfwave_max(float x) {
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float halfwave_sum(float x) {
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+// Fill an AttnArgs from the public struct; validates what both directions share.
+int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a);
+
+}  // namespace rswa

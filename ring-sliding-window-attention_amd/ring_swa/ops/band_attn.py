@@ -1,0 +1,212 @@
+"""Kernel-level attention operators: one masked block, forward or backward.
+
+These take the place of the flash-attn wrappers of the upstream package
+(``ring_swa/ops/wrap_flash.py:168-429``) and keep their names, positional
+argument order and conventions:
+
+* ``window_size = (left, right)``, ``-1`` = unbounded, bottom-right aligned;
+  ``causal=True`` forces ``right = 0``;
+* forward returns ``(out, softmax_lse)`` with ``softmax_lse`` fp32
+  ``[batch, heads, seq]`` (dense) or ``[heads, total]`` (packed);
+* backward writes into the caller's ``dq, dk, dv`` and uses the caller's
+  ``o`` / ``softmax_lse`` (which may be merged statistics).
+
+Additions (keyword-only): ``num_sink`` (attention-sink keys at the head of each
+sequence, visible regardless of the left window bound).  Rows without any
+visible key produce ``out = 0``, ``lse = -inf`` (the merge identity).
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from .. import _lib
+
+
+def _check_qkv(q, k, v, packed: bool):
+    nd = 3 if packed else 4
+    assert q.dim() == nd and k.dim() == nd and v.dim() == nd, (
+        f"expected {nd}-d q/k/v, got {q.dim()}, {k.dim()}, {v.dim()}"
+    )
+    assert k.shape == v.shape, "k and v must have the same shape"
+    assert q.shape[-1] == k.shape[-1], "head_dim mismatch"
+    assert q.dtype == k.dtype == v.dtype, "q, k, v must share a dtype"
+    assert q.shape[-2] % k.shape[-2] == 0, (
+        "Number of query heads must be divisible by number of key/value heads"
+    )
+    if not packed:
+        assert q.shape[0] == k.shape[0], "batch mismatch"
+    for t in (q, k, v):
+        assert t.stride(-1) == 1, "last dimension must be contiguous"
+
+
+def _strides3(t: torch.Tensor, packed: bool):
+    if packed:
+        return (0, t.stride(0), t.stride(1))
+    return (t.stride(0), t.stride(1), t.stride(2))
+
+
+def _lse_strides(lse: torch.Tensor, packed: bool):
+    if packed:
+        return (0, lse.stride(0), lse.stride(1))
+    return (lse.stride(0), lse.stride(1), lse.stride(2))
+
+
+def _params(q, k, v, softmax_scale, window_size, causal, cu_q, cu_k, num_sink) -> "_lib.AttnParams":
+    packed = cu_q is not None
+    p = _lib.AttnParams()
+    p.dtype = _lib.dtype_code(q)
+    p.head_dim = q.shape[-1]
+    p.heads_q = q.shape[-2]
+    p.heads_kv = k.shape[-2]
+    if packed:
+        assert cu_k is not None, "cu_seqlens_k is required with cu_seqlens_q"
+        for cu in (cu_q, cu_k):
+            assert cu.dtype == torch.int32 and cu.dim() == 1 and cu.is_contiguous(), (
+                "cu_seqlens must be a contiguous 1-d int32 tensor"
+            )
+            assert cu.device == q.device, "cu_seqlens must live on the tensors' device"
+        assert cu_q.numel() == cu_k.numel() and cu_q.numel() >= 2
+        p.batch = cu_q.numel() - 1
+        p.total_q, p.total_k = q.shape[0], k.shape[0]
+        # only upper bounds are needed, so no device->host read of the lengths
+        p.seqlen_q, p.seqlen_k = q.shape[0], k.shape[0]
+        p.cu_seqlens_q, p.cu_seqlens_k = cu_q.data_ptr(), cu_k.data_ptr()
+    else:
+        p.batch = q.shape[0]
+        p.seqlen_q, p.seqlen_k = q.shape[1], k.shape[1]
+        p.total_q = p.total_k = 0
+        p.cu_seqlens_q = p.cu_seqlens_k = None
+    p.softmax_scale = float(softmax_scale)
+    p.window_left, p.window_right = int(window_size[0]), int(window_size[1])
+    p.causal = 1 if causal else 0
+    p.num_sink = int(num_sink)
+    p.q, p.k, p.v = q.data_ptr(), k.data_ptr(), v.data_ptr()
+    p.q_stride = _lib.i64x3(_strides3(q, packed))
+    p.k_stride = _lib.i64x3(_strides3(k, packed))
+    p.v_stride = _lib.i64x3(_strides3(v, packed))
+    return p
+
+
+def attn_fwd(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    softmax_scale: Optional[float],
+    window_size: Tuple[int, int] = (-1, -1),
+    causal: bool = False,
+    cu_seqlens_q: Optional[torch.Tensor] = None,
+    cu_seqlens_k: Optional[torch.Tensor] = None,
+    *,
+    num_sink: int = 0,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Masked attention forward on the HIP kernel; returns ``(out, lse)``."""
+    packed = cu_seqlens_q is not None
+    _check_qkv(q, k, v, packed)
+    dev = _lib.require_device(q, k, v)
+    if softmax_scale is None:
+        softmax_scale = q.shape[-1] ** (-0.5)
+    out = torch.empty(q.shape, dtype=q.dtype, device=dev)
+    if packed:
+        lse = torch.empty((q.shape[1], q.shape[0]), dtype=torch.float32, device=dev)
+    else:
+        lse = torch.empty((q.shape[0], q.shape[2], q.shape[1]), dtype=torch.float32, device=dev)
+    if q.numel() == 0:
+        return out, lse
+    p = _params(q, k, v, softmax_scale, window_size, causal, cu_seqlens_q, cu_seqlens_k, num_sink)
+    p.out = out.data_ptr()
+    p.out_stride = _lib.i64x3(_strides3(out, packed))
+    p.lse = lse.data_ptr()
+    p.lse_stride = _lib.i64x3(_lse_strides(lse, packed))
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().rswa_attn_fwd(p, _lib.stream_ptr(dev)))
+    return out, lse
+
+
+def attn_bwd(
+    q, k, v, o, softmax_lse, do, dq, dk, dv,
+    softmax_scale: Optional[float],
+    window_size: Tuple[int, int] = (-1, -1),
+    causal: bool = False,
+    cu_seqlens_q: Optional[torch.Tensor] = None,
+    cu_seqlens_k: Optional[torch.Tensor] = None,
+    *,
+    num_sink: int = 0,
+) -> None:
+    """Masked attention backward; overwrites ``dq, dk, dv`` (views are fine)."""
+    packed = cu_seqlens_q is not None
+    _check_qkv(q, k, v, packed)
+    dev = _lib.require_device(q, k, v, o, softmax_lse, do, dq, dk, dv)
+    assert o.shape == q.shape and do.shape == q.shape and dq.shape == q.shape
+    assert dk.shape == k.shape and dv.shape == v.shape
+    assert o.dtype == q.dtype and do.dtype == q.dtype
+    assert dq.dtype == q.dtype and dk.dtype == q.dtype and dv.dtype == q.dtype, (
+        "dq, dk, dv must have the dtype of q"
+    )
+    assert softmax_lse.dtype == torch.float32, "softmax_lse must be fp32"
+    for t in (o, do, dq, dk, dv):
+        assert t.stride(-1) == 1, "last dimension must be contiguous"
+    if packed:
+        assert softmax_lse.shape == (q.shape[1], q.shape[0])
+    else:
+        assert softmax_lse.shape == (q.shape[0], q.shape[2], q.shape[1])
+    if softmax_scale is None:
+        softmax_scale = q.shape[-1] ** (-0.5)
+    if q.numel() == 0 or k.numel() == 0:
+        dq.zero_()
+        dk.zero_()
+        dv.zero_()
+        return
+    p = _params(q, k, v, softmax_scale, window_size, causal, cu_seqlens_q, cu_seqlens_k, num_sink)
+    p.out = o.data_ptr()
+    p.out_stride = _lib.i64x3(_strides3(o, packed))
+    p.lse = softmax_lse.data_ptr()
+    p.lse_stride = _lib.i64x3(_lse_strides(softmax_lse, packed))
+    p.dout = do.data_ptr()
+    p.dout_stride = _lib.i64x3(_strides3(do, packed))
+    p.dq, p.dk, p.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
+    p.dq_stride = _lib.i64x3(_strides3(dq, packed))
+    p.dk_stride = _lib.i64x3(_strides3(dk, packed))
+    p.dv_stride = _lib.i64x3(_strides3(dv, packed))
+    L = _lib.lib()
+    need = int(L.rswa_attn_bwd_workspace_bytes(p))
+    ws = torch.empty(need, dtype=torch.uint8, device=dev)  # caching allocator: 512-B aligned
+    p.workspace = ws.data_ptr()
+    p.workspace_bytes = need
+    with torch.cuda.device(dev):
+        _lib.check(L.rswa_attn_bwd(p, _lib.stream_ptr(dev)))
+
+
+# ---- names of the upstream wrappers -----------------------------------------
+def wrapped_flash_attn_fwd(q, k, v, softmax_scale, window_size, causal, *, num_sink=0):
+    """Dense forward, ``ring_swa/ops/wrap_flash.py:168``: returns ``(out, softmax_lse)``."""
+    return attn_fwd(q, k, v, softmax_scale, window_size, causal, num_sink=num_sink)
+
+
+def wrapped_flash_attn_fwd_varlen(
+    q, k, v, softmax_scale, window_size, cu_seqlens_q, cu_seqlens_k,
+    max_seqlen_q=None, max_seqlen_k=None, causal=False, *, num_sink=0,
+):
+    """Packed forward, ``ring_swa/ops/wrap_flash.py:203``.  ``max_seqlen_*`` are
+    accepted for signature compatibility and unused (no host sync is needed)."""
+    return attn_fwd(q, k, v, softmax_scale, window_size, causal, cu_seqlens_q, cu_seqlens_k,
+                    num_sink=num_sink)
+
+
+def wrapped_flash_attn_bwd(
+    q, k, v, o, softmax_lse, do, dq, dk, dv, softmax_scale, window_size, causal, *, num_sink=0
+):
+    """Dense backward, ``ring_swa/ops/wrap_flash.py:276``; fills ``dq, dk, dv``."""
+    attn_bwd(q, k, v, o, softmax_lse, do, dq, dk, dv, softmax_scale, window_size, causal,
+             num_sink=num_sink)
+
+
+def wrapped_flash_attn_bwd_varlen(
+    q, k, v, o, softmax_lse, do, dq, dk, dv, softmax_scale, window_size,
+    cu_seqlens_q, cu_seqlens_k, max_seqlen_q=None, max_seqlen_k=None, causal=False, *,
+    num_sink=0,
+):
+    """Packed backward, ``ring_swa/ops/wrap_flash.py:330``; fills ``dq, dk, dv``."""
+    attn_bwd(q, k, v, o, softmax_lse, do, dq, dk, dv, softmax_scale, window_size, causal,
+             cu_seqlens_q, cu_seqlens_k, num_sink=num_sink)

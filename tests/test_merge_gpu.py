@@ -104,7 +104,8 @@ def test_merge_rejects_bad_arguments():
     o, l, on, ln = (t.cuda() for t in _mk(1, 8, 2, 128, *DT["ring"]))
     with pytest.raises(AssertionError):
         merge_attn_out(o, l.transpose(1, 2), on, ln)
+    wide = torch.zeros(1, 8, 2, 256, device="cuda")[..., ::2]  # dim stride 2
     with pytest.raises(NotImplementedError):
-        merge_attn_out(o.transpose(2, 3), l, on.transpose(2, 3), ln)  # dim stride != 1
+        merge_attn_out(wide, l, on, ln)
     with pytest.raises(RuntimeError):
         merge_attn_out(o.cpu(), l.cpu(), on.cpu(), ln.cpu())
