@@ -86,6 +86,7 @@ int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a) {
     a.do_st[0] = a.dq_st[0] = a.dk_st[0] = a.dv_st[0] = 0;
   }
   a.rows_q = packed ? p->total_q : (int64_t)p->batch * p->seqlen_q;
+  a.rows_k = packed ? p->total_k : (int64_t)p->batch * p->seqlen_k;
   a.batch = p->batch;
   a.heads_q = p->heads_q;
   a.heads_kv = p->heads_kv;

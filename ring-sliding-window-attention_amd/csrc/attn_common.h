@@ -35,6 +35,7 @@ struct AttnArgs {
   const int32_t* cu_k;
   int64_t q_st[3], k_st[3], v_st[3], o_st[3], do_st[3], dq_st[3], dk_st[3], dv_st[3], lse_st[3];
   int64_t rows_q;  // batch * seqlen_q (dense) or total_q (packed)
+  int64_t rows_k;  // batch * seqlen_k (dense) or total_k (packed)
   int32_t batch, heads_q, heads_kv, group;  // group = heads_q / heads_kv
   int32_t seqlen_q, seqlen_k;
   int32_t wl, wr, n_sink;  // wl/wr < 0: unbounded

@@ -1,0 +1,230 @@
+"""GPU parity of the HIP backward attention kernels (through the C ABI) against
+the CPU oracle.  Tolerance stated for this path: dQ, dK, dV within 5e-2 in
+relative norm ||x - ref|| / ||ref||."""
+import itertools
+
+import pytest
+import torch
+
+from oracle import attention_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+GRAD_TOL = 5e-2
+
+
+def _rand(shape, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(*shape, generator=g).to(dtype)
+
+
+def _relnorm(x, ref):
+    x = x.float().cpu()
+    assert not torch.isnan(x).any()
+    den = ref.norm().item()
+    if den == 0.0:
+        return x.norm().item()
+    return (x - ref).norm().item() / den
+
+
+def _run_dense(q, k, v, do, scale, window, causal, ns):
+    """fwd + bwd on the GPU kernels, dq/dk/dv into fresh buffers."""
+    from ring_swa.ops import wrapped_flash_attn_bwd, wrapped_flash_attn_fwd
+
+    dq_, dk_, dv_, ddo = q.cuda(), k.cuda(), v.cuda(), do.cuda()
+    out, lse = wrapped_flash_attn_fwd(dq_, dk_, dv_, scale, window, causal, num_sink=ns)
+    gq = torch.full_like(dq_, float("nan"))
+    gk = torch.full_like(dk_, float("nan"))
+    gv = torch.full_like(dv_, float("nan"))
+    wrapped_flash_attn_bwd(dq_, dk_, dv_, out, lse, ddo, gq, gk, gv, scale, window, causal,
+                           num_sink=ns)
+    torch.cuda.synchronize()
+    return out, lse, gq, gk, gv
+
+
+DENSE_CASES = [
+    # (B, Sq, Sk, Hq, Hkv, D, window, causal, n_sink)
+    (1, 100, 100, 8, 2, 64, (50, 50), False, 0),     # test/test_local_swa.py:98-141
+    (1, 1024, 1024, 8, 2, 64, (128, 0), True, 1),    # test/test_local_slm.py:76-119
+    (2, 300, 300, 4, 4, 128, (37, 0), True, 0),
+    (1, 257, 257, 4, 1, 128, (-1, -1), False, 0),
+    (1, 130, 130, 2, 2, 128, (0, 0), True, 0),
+    (1, 200, 333, 4, 2, 128, (40, 0), True, 0),
+    (1, 333, 200, 4, 2, 128, (40, 0), True, 0),      # leading rows see nothing
+    (1, 96, 160, 2, 1, 128, (0, 4096), False, 0),
+    (1, 160, 160, 2, 1, 128, (70, 160), False, 0),
+    (1, 190, 64, 2, 1, 128, (10, 4096), False, 0),
+    (2, 700, 700, 4, 2, 128, (100, 0), True, 4),
+    (1, 513, 513, 2, 2, 128, (1000, 0), True, 2),
+    (1, 2048, 2048, 4, 2, 128, (500, 0), True, 0),
+    (1, 1, 1, 1, 1, 128, (5, 0), True, 0),
+]
+
+
+@pytest.mark.parametrize("case", DENSE_CASES, ids=lambda c: "x".join(str(x) for x in c))
+def test_bwd_dense_matches_oracle(case):
+    b, sq, sk, hq, hk, d, window, causal, ns = case
+    q = _rand((b, sq, hq, d), torch.bfloat16, 1)
+    k = _rand((b, sk, hk, d), torch.bfloat16, 2)
+    v = _rand((b, sk, hk, d), torch.bfloat16, 3)
+    do = _rand((b, sq, hq, d), torch.bfloat16, 4)
+    scale = d ** -0.5
+    _, _, rq, rk, rv = O.attention_fwd_bwd(
+        lambda q, k, v: O.window_attention(q, k, v, scale, window, causal, ns), q, k, v, do
+    )
+    out, lse, gq, gk, gv = _run_dense(q, k, v, do, scale, window, causal, ns)
+    errs = [_relnorm(g, r) for g, r in ((gq, rq), (gk, rk), (gv, rv))]
+    assert max(errs) <= GRAD_TOL, f"rel-norm errors dq/dk/dv = {errs}"
+
+
+def test_bwd_with_ones_upstream_like_the_reference_test():
+    """dO = ones, GQA 4:1, two-sided window — the check of test/test_local_swa.py:129-141."""
+    q = _rand((1, 100, 8, 64), torch.bfloat16, 42)
+    k = _rand((1, 100, 2, 64), torch.bfloat16, 43)
+    v = _rand((1, 100, 2, 64), torch.bfloat16, 44)
+    do = torch.ones(1, 100, 8, 64, dtype=torch.bfloat16)
+    _, _, rq, rk, rv = O.attention_fwd_bwd(
+        lambda q, k, v: O.window_attention(q, k, v, None, (50, 50), False), q, k, v, do
+    )
+    _, _, gq, gk, gv = _run_dense(q, k, v, do, 64 ** -0.5, (50, 50), False, 0)
+    for g, r in ((gq, rq), (gk, rk), (gv, rv)):
+        # the reference asserts atol = rtol = 1e-2 on bf16 gradients
+        bad = (g.float().cpu() - r).abs() > 1e-2 + 1e-2 * r.abs()
+        assert bad.float().mean().item() < 1e-2, "too many elements outside atol=rtol=1e-2"
+        assert _relnorm(g, r) <= GRAD_TOL
+
+
+def test_bwd_uses_the_callers_merged_statistics():
+    """Keys split in two blocks, each backward fed the FINAL (o, lse): the sum equals
+    the gradient of attention over all keys (ring_swa/sliding_window/nonvarlen.py:242-253)."""
+    from ring_swa.ops import merge_attn_out, wrapped_flash_attn_bwd, wrapped_flash_attn_fwd
+
+    b, s, hq, hk, d, w = 1, 384, 4, 2, 128, 200
+    q = _rand((b, s, hq, d), torch.bfloat16, 1)
+    k = _rand((b, 2 * s, hk, d), torch.bfloat16, 2)
+    v = _rand((b, 2 * s, hk, d), torch.bfloat16, 3)
+    do = _rand((b, s, hq, d), torch.bfloat16, 4)
+    # queries are the last s positions of a 2s-long sequence, window w: keys split at s
+    _, _, rq, rk, rv = O.attention_fwd_bwd(
+        lambda q, k, v: O.window_attention(q, k, v, None, (w, 0), True), q, k, v, do
+    )
+    dq_, dk_, dv_, ddo = q.cuda(), k.cuda(), v.cuda(), do.cuda()
+    # block A: own chunk (causal band); block B: previous chunk, upper-right triangle
+    oa, la = wrapped_flash_attn_fwd(dq_, dk_[:, s:], dv_[:, s:], None, (w, 0), True)
+    ob, lb = wrapped_flash_attn_fwd(dq_[:, :w], dk_[:, s - w:s], dv_[:, s - w:s], None, (0, s), False)
+    acc = oa.float()
+    lacc = la.clone()
+    merge_attn_out(acc[:, :w], lacc[:, :, :w], ob, lb)
+    o_fin = acc.to(torch.bfloat16)
+    gq = torch.zeros_like(dq_, dtype=torch.float32)
+    gk = torch.zeros_like(dk_, dtype=torch.float32)
+    gv = torch.zeros_like(dv_, dtype=torch.float32)
+    tq, tk, tv = torch.empty_like(dq_), torch.empty_like(dk_[:, s:]), torch.empty_like(dv_[:, s:])
+    wrapped_flash_attn_bwd(dq_, dk_[:, s:], dv_[:, s:], o_fin, lacc, ddo, tq, tk, tv, None, (w, 0), True)
+    gq += tq
+    gk[:, s:] += tk
+    gv[:, s:] += tv
+    tq2 = torch.empty_like(dq_[:, :w])
+    tk2, tv2 = torch.empty_like(dk_[:, s - w:s]), torch.empty_like(dv_[:, s - w:s])
+    wrapped_flash_attn_bwd(dq_[:, :w], dk_[:, s - w:s], dv_[:, s - w:s], o_fin[:, :w],
+                           lacc[:, :, :w].contiguous(), ddo[:, :w], tq2, tk2, tv2, None, (0, s), False)
+    gq[:, :w] += tq2
+    gk[:, s - w:s] += tk2
+    gv[:, s - w:s] += tv2
+    torch.cuda.synchronize()
+    errs = [_relnorm(g, r) for g, r in ((gq, rq), (gk, rk), (gv, rv))]
+    assert max(errs) <= GRAD_TOL, f"rel-norm errors dq/dk/dv = {errs}"
+
+
+def test_bwd_into_strided_views():
+    """dq/dk/dv handed in as slices of larger buffers (ring_swa/streaming_llm/naive.py:53-66)."""
+    from ring_swa.ops import wrapped_flash_attn_bwd, wrapped_flash_attn_fwd
+
+    q = _rand((2, 201, 4, 128), torch.bfloat16, 1)
+    k = _rand((2, 201, 2, 128), torch.bfloat16, 2)
+    v = _rand((2, 201, 2, 128), torch.bfloat16, 3)
+    do = _rand((2, 201, 4, 128), torch.bfloat16, 4)
+    _, _, rq, rk, rv = O.attention_fwd_bwd(
+        lambda q, k, v: O.window_attention(q, k, v, None, (20, 0), True),
+        q[:, 1:], k[:, 1:], v[:, 1:], do[:, 1:],
+    )
+    dq_, dk_, dv_, ddo = q.cuda(), k.cuda(), v.cuda(), do.cuda()
+    o, lse = wrapped_flash_attn_fwd(dq_[:, 1:], dk_[:, 1:], dv_[:, 1:], None, (20, 0), True)
+    gq, gk, gv = torch.zeros_like(dq_), torch.zeros_like(dk_), torch.zeros_like(dv_)
+    wrapped_flash_attn_bwd(dq_[:, 1:], dk_[:, 1:], dv_[:, 1:], o, lse, ddo[:, 1:], gq[:, 1:],
+                           gk[:, 1:], gv[:, 1:], None, (20, 0), True)
+    torch.cuda.synchronize()
+    assert torch.all(gq[:, 0] == 0) and torch.all(gk[:, 0] == 0) and torch.all(gv[:, 0] == 0)
+    errs = [_relnorm(g[:, 1:], r) for g, r in ((gq, rq), (gk, rk), (gv, rv))]
+    assert max(errs) <= GRAD_TOL, f"rel-norm errors dq/dk/dv = {errs}"
+
+
+@pytest.mark.parametrize("lens,window,ns", [
+    ([5, 130, 64, 1, 300], (50, 0), 0),
+    ([257, 255], (-1, 0), 0),
+    ([100, 400, 129], (64, 0), 4),
+])
+def test_bwd_varlen_matches_oracle(lens, window, ns):
+    from ring_swa.ops import wrapped_flash_attn_bwd_varlen, wrapped_flash_attn_fwd_varlen
+
+    cu = torch.tensor([0] + list(itertools.accumulate(lens)), dtype=torch.int32)
+    t = int(cu[-1])
+    q = _rand((t, 4, 128), torch.bfloat16, 1)
+    k = _rand((t, 2, 128), torch.bfloat16, 2)
+    v = _rand((t, 2, 128), torch.bfloat16, 3)
+    do = _rand((t, 4, 128), torch.bfloat16, 4)
+    _, _, rq, rk, rv = O.attention_fwd_bwd(
+        lambda q, k, v: O.window_attention_varlen(q, k, v, cu, cu, None, window, True, ns),
+        q, k, v, do,
+    )
+    dq_, dk_, dv_, ddo, dcu = q.cuda(), k.cuda(), v.cuda(), do.cuda(), cu.cuda()
+    o, lse = wrapped_flash_attn_fwd_varlen(dq_, dk_, dv_, None, window, dcu, dcu, None, None, True,
+                                           num_sink=ns)
+    gq, gk, gv = torch.empty_like(dq_), torch.empty_like(dk_), torch.empty_like(dv_)
+    wrapped_flash_attn_bwd_varlen(dq_, dk_, dv_, o, lse, ddo, gq, gk, gv, None, window, dcu, dcu,
+                                  None, None, True, num_sink=ns)
+    torch.cuda.synchronize()
+    errs = [_relnorm(g, r) for g, r in ((gq, rq), (gk, rk), (gv, rv))]
+    assert max(errs) <= GRAD_TOL, f"rel-norm errors dq/dk/dv = {errs}"
+
+
+def test_bwd_varlen_one_key_per_sequence():
+    """The per-sequence sink backward of ring_swa/streaming_llm/naive.py:181-206: every
+    sequence attends one key of its own (cu_seqlens_k = arange)."""
+    from ring_swa.ops import wrapped_flash_attn_bwd_varlen, wrapped_flash_attn_fwd_varlen
+
+    lens_q = [70, 200, 3]
+    cu_q = torch.tensor([0] + list(itertools.accumulate(lens_q)), dtype=torch.int32)
+    cu_k = torch.arange(0, 4, dtype=torch.int32)
+    t = int(cu_q[-1])
+    q = _rand((t, 4, 128), torch.bfloat16, 1)
+    k = _rand((3, 2, 128), torch.bfloat16, 2)
+    v = _rand((3, 2, 128), torch.bfloat16, 3)
+    do = _rand((t, 4, 128), torch.bfloat16, 4)
+    _, _, rq, rk, rv = O.attention_fwd_bwd(
+        lambda q, k, v: O.window_attention_varlen(q, k, v, cu_q, cu_k, None, (-1, -1), False),
+        q, k, v, do,
+    )
+    dq_, dk_, dv_, ddo = q.cuda(), k.cuda(), v.cuda(), do.cuda()
+    o, lse = wrapped_flash_attn_fwd_varlen(dq_, dk_, dv_, None, (-1, -1), cu_q.cuda(), cu_k.cuda(),
+                                           200, 1, False)
+    gq, gk, gv = torch.empty_like(dq_), torch.empty_like(dk_), torch.empty_like(dv_)
+    wrapped_flash_attn_bwd_varlen(dq_, dk_, dv_, o, lse, ddo, gq, gk, gv, None, (-1, -1),
+                                  cu_q.cuda(), cu_k.cuda(), 200, 1, False)
+    torch.cuda.synchronize()
+    # softmax over a single key is constant: dq and dk vanish, dv is the column sum of dO
+    assert gq.abs().max().item() <= 1e-2 and gk.abs().max().item() <= 1e-2
+    assert _relnorm(gv, rv) <= GRAD_TOL
+
+
+def test_bwd_fp16():
+    q = _rand((1, 150, 4, 128), torch.float16, 1)
+    k = _rand((1, 150, 2, 128), torch.float16, 2)
+    v = _rand((1, 150, 2, 128), torch.float16, 3)
+    do = _rand((1, 150, 4, 128), torch.float16, 4)
+    _, _, rq, rk, rv = O.attention_fwd_bwd(
+        lambda q, k, v: O.window_attention(q, k, v, 0.2, (33, 0), True), q, k, v, do
+    )
+    _, _, gq, gk, gv = _run_dense(q, k, v, do, 0.2, (33, 0), True, 0)
+    errs = [_relnorm(g, r) for g, r in ((gq, rq), (gk, rk), (gv, rv))]
+    assert max(errs) <= GRAD_TOL, f"rel-norm errors dq/dk/dv = {errs}"
