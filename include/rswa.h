@@ -94,6 +94,10 @@ int rswa_merge_attn_out(void* o, int o_dtype, const int64_t* o_stride,
  * where a negative window bound means unbounded and causal != 0 forces
  * window_right = 0.  num_sink > 0 additionally makes keys j < num_sink visible
  * whenever they satisfy the right bound (attention sinks at the sequence head).
+ * shift_explicit != 0 replaces the bottom-right shift by the caller's `shift`
+ * (any sign) for every sequence: e.g. shift = 0 aligns the diagonals top-left,
+ * and shift = -(w + 1) with window_left < 0, window_right = 0 selects the keys
+ * that lie more than w positions behind the query.
  * Rows with no visible key produce out = 0, lse = -inf.
  *
  * lse is the natural-log sum of exp(softmax_scale * q.k) over visible keys.
@@ -125,6 +129,8 @@ typedef struct rswa_attn_params {
   int32_t window_right; /* < 0: unbounded */
   int32_t causal;
   int32_t num_sink;
+  int32_t shift_explicit; /* 0: shift = len_k - len_q (flash-attn alignment) */
+  int32_t shift;          /* used when shift_explicit != 0                   */
 
   const void* q;
   const void* k;

@@ -96,6 +96,8 @@ int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a) {
   a.wl = p->window_left < 0 ? -1 : p->window_left;
   a.wr = p->causal ? 0 : (p->window_right < 0 ? -1 : p->window_right);
   a.n_sink = p->num_sink;
+  a.shift_explicit = p->shift_explicit != 0;
+  a.shift_val = p->shift;
   a.n_tile = 0;
   a.n_work = 0;
   a.scale = p->softmax_scale;

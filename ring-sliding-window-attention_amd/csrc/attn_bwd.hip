@@ -96,7 +96,7 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(const AttnArgs a) {
   const int j0 = kt * C::BN;
   if (j0 >= len_k) return;
   const int j_last = min(j0 + C::BN, len_k) - 1;
-  const int shift = len_k - len_q;
+  const int shift = a.shift_explicit ? a.shift_val : len_k - len_q;
 
   const T* k_ptr = (const T*)a.k + b * a.k_st[0] + s.k_row0 * a.k_st[1] + hk * a.k_st[2];
   const T* v_ptr = (const T*)a.v + b * a.v_st[0] + s.k_row0 * a.v_st[1] + hk * a.v_st[2];

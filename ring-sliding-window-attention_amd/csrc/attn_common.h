@@ -39,6 +39,7 @@ struct AttnArgs {
   int32_t batch, heads_q, heads_kv, group;  // group = heads_q / heads_kv
   int32_t seqlen_q, seqlen_k;
   int32_t wl, wr, n_sink;  // wl/wr < 0: unbounded
+  int32_t shift_explicit, shift_val;
   int32_t n_tile;          // tiles per sequence (dense) / total tile slots (packed)
   int32_t n_work;          // logical blocks
   float scale, scale_log2;
@@ -70,7 +71,7 @@ struct RowBounds {
 
 __device__ __forceinline__ RowBounds row_bounds(const AttnArgs& a, int i, int len_q, int len_k) {
   RowBounds r;
-  const int shift = len_k - len_q;
+  const int shift = a.shift_explicit ? a.shift_val : len_k - len_q;
   r.hi = (a.wr >= 0) ? min(len_k - 1, i + shift + a.wr) : len_k - 1;
   r.lo = (a.wl >= 0) ? max(0, i + shift - a.wl) : 0;
   if (i >= len_q) r.hi = -1;  // rows past the end see nothing

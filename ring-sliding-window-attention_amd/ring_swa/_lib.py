@@ -47,6 +47,8 @@ class AttnParams(Structure):
         ("window_right", c_int32),
         ("causal", c_int32),
         ("num_sink", c_int32),
+        ("shift_explicit", c_int32),
+        ("shift", c_int32),
         ("q", c_void_p),
         ("k", c_void_p),
         ("v", c_void_p),

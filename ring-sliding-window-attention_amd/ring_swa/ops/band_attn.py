@@ -12,7 +12,9 @@ argument order and conventions:
   ``o`` / ``softmax_lse`` (which may be merged statistics).
 
 Additions (keyword-only): ``num_sink`` (attention-sink keys at the head of each
-sequence, visible regardless of the left window bound).  Rows without any
+sequence, visible regardless of the left window bound) and, on ``attn_fwd`` /
+``attn_bwd``, ``mask_shift`` (explicit diagonal offset replacing the bottom-right
+``len_k - len_q``).  Rows without any
 visible key produce ``out = 0``, ``lse = -inf`` (the merge identity).
 """
 from __future__ import annotations
@@ -53,7 +55,8 @@ def _lse_strides(lse: torch.Tensor, packed: bool):
     return (lse.stride(0), lse.stride(1), lse.stride(2))
 
 
-def _params(q, k, v, softmax_scale, window_size, causal, cu_q, cu_k, num_sink) -> "_lib.AttnParams":
+def _params(q, k, v, softmax_scale, window_size, causal, cu_q, cu_k, num_sink,
+            mask_shift=None) -> "_lib.AttnParams":
     packed = cu_q is not None
     p = _lib.AttnParams()
     p.dtype = _lib.dtype_code(q)
@@ -82,6 +85,8 @@ def _params(q, k, v, softmax_scale, window_size, causal, cu_q, cu_k, num_sink) -
     p.window_left, p.window_right = int(window_size[0]), int(window_size[1])
     p.causal = 1 if causal else 0
     p.num_sink = int(num_sink)
+    p.shift_explicit = 0 if mask_shift is None else 1
+    p.shift = 0 if mask_shift is None else int(mask_shift)
     p.q, p.k, p.v = q.data_ptr(), k.data_ptr(), v.data_ptr()
     p.q_stride = _lib.i64x3(_strides3(q, packed))
     p.k_stride = _lib.i64x3(_strides3(k, packed))
@@ -100,6 +105,7 @@ def attn_fwd(
     cu_seqlens_k: Optional[torch.Tensor] = None,
     *,
     num_sink: int = 0,
+    mask_shift: Optional[int] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     """Masked attention forward on the HIP kernel; returns ``(out, lse)``."""
     packed = cu_seqlens_q is not None
@@ -114,7 +120,8 @@ def attn_fwd(
         lse = torch.empty((q.shape[0], q.shape[2], q.shape[1]), dtype=torch.float32, device=dev)
     if q.numel() == 0:
         return out, lse
-    p = _params(q, k, v, softmax_scale, window_size, causal, cu_seqlens_q, cu_seqlens_k, num_sink)
+    p = _params(q, k, v, softmax_scale, window_size, causal, cu_seqlens_q, cu_seqlens_k, num_sink,
+                mask_shift)
     p.out = out.data_ptr()
     p.out_stride = _lib.i64x3(_strides3(out, packed))
     p.lse = lse.data_ptr()
@@ -133,6 +140,7 @@ def attn_bwd(
     cu_seqlens_k: Optional[torch.Tensor] = None,
     *,
     num_sink: int = 0,
+    mask_shift: Optional[int] = None,
 ) -> None:
     """Masked attention backward; overwrites ``dq, dk, dv`` (views are fine)."""
     packed = cu_seqlens_q is not None
@@ -158,7 +166,8 @@ def attn_bwd(
         dk.zero_()
         dv.zero_()
         return
-    p = _params(q, k, v, softmax_scale, window_size, causal, cu_seqlens_q, cu_seqlens_k, num_sink)
+    p = _params(q, k, v, softmax_scale, window_size, causal, cu_seqlens_q, cu_seqlens_k, num_sink,
+                mask_shift)
     p.out = o.data_ptr()
     p.out_stride = _lib.i64x3(_strides3(o, packed))
     p.lse = softmax_lse.data_ptr()

@@ -1,0 +1,248 @@
+"""One context-parallel rank's share of ring sliding-window attention, on one GPU.
+
+The compute body of upstream's ring loops
+(``ring_swa/sliding_window/nonvarlen.py:46-150`` forward, ``:182-333`` backward;
+``ring_swa/sliding_window/varlen.py:56-172`` and ``:194-359``) with the P2P
+exchange replaced by KV chunks the caller already holds in HBM: the rank's own
+chunk plus the chunks of the ranks before it.  Per step: one band-attention
+kernel on the block the window selects, LSE-merged into the running output;
+backward runs one kernel call per block with the final merged ``(o, lse)`` and
+accumulates ``dq`` / per-chunk ``dkv`` in fp32, as upstream does.
+
+What is left out is exactly what needs a second GPU: moving KV forward and
+KV + dKV backward around the ring.
+"""
+from __future__ import annotations
+
+import math
+from typing import List, Optional, Sequence, Tuple
+
+import torch
+
+from .ops.band_attn import attn_bwd, attn_fwd
+from .ops.lse_merge import merge_attn_out
+
+Step = Tuple[int, slice, slice, Tuple[int, int], bool]
+
+
+def ring_comm_times(window_size: int, seq_len: int, cp_size: int) -> int:
+    """Number of KV hops a rank needs: ``min(ceil(w / S), cp_size - 1)``
+    (``ring_swa/sliding_window/nonvarlen.py:46-49``)."""
+    return min(math.ceil(window_size / seq_len), cp_size - 1)
+
+
+def plan_nonvarlen(seq_len: int, window_size: int, cp_size: int, rank: int) -> List[Step]:
+    """Blocks of one rank as ``(step, q_slice, kv_slice, (left, right), causal)``.
+
+    Step ``i`` pairs the rank's queries with the chunk of rank ``rank - i``; the
+    four block shapes are those of ``ring_swa/sliding_window/nonvarlen.py:95-150``
+    (diagonal / full / lower-left corner cut / upper-right corner only).
+    Wrap-around steps are dropped (``:97``).
+    """
+    s, w = seq_len, window_size
+    plan: List[Step] = []
+    whole = slice(0, s)
+    for i in range(ring_comm_times(w, s, cp_size) + 1):
+        if rank - i < 0:
+            continue
+        if i == 0:
+            plan.append((0, whole, whole, (w, 0), True))
+        elif (i + 1) * s <= w + 1:
+            plan.append((i, whole, whole, (-1, -1), False))
+        elif i * s < w + 1:
+            plan.append((i, whole, whole, (w % s, s), False))
+        elif (i - 1) * s < w < i * s:
+            v = w % s
+            plan.append((i, slice(0, v), slice(s - v, s), (0, s), False))
+        else:
+            raise ValueError(f"[forward] Invalid step: {i}")
+    return plan
+
+
+def plan_varlen(cu_seqlens: Sequence[int], seq_len: int, window_size: int, cp_size: int,
+                rank: int) -> Tuple[List[int], List[Step]]:
+    """Packed twin (``ring_swa/sliding_window/varlen.py:56-74,127-172``).
+
+    Returns the rank-local ``cu_seqlens`` of the diagonal block and the plan; only
+    the rank's first sequence (the one that may start on an earlier rank) has
+    off-diagonal blocks, each a dense rectangle.
+    """
+    cu = [int(c) for c in cu_seqlens]
+    s, w = seq_len, window_size
+    start, end = rank * s, (rank + 1) * s
+    first = min(i for i, c in enumerate(cu) if c > start)
+    last = min(i for i, c in enumerate(cu) if c >= end)
+    local_cu = [0] + [c - start for c in cu[first:last]] + [s]
+    first_q_len = local_cu[1]
+    first_kv_len = start - cu[first - 1]
+    plan: List[Step] = [(0, slice(0, s), slice(0, s), (w, 0), True)]
+    for i in range(1, ring_comm_times(w, s, cp_size) + 1):
+        if rank - i < 0:
+            continue
+        if min(first_kv_len, w) > (i - 1) * s:
+            vw = min(w - (i - 1) * s, 2 * s)
+            vk = min(first_kv_len - (i - 1) * s, s, vw)
+            vq = min(first_q_len, vw)
+            plan.append((i, slice(0, vq), slice(s - vk, s), (vw - vq, s), False))
+    return local_cu, plan
+
+
+class RankShareFunc(torch.autograd.Function):
+    """Dense tensors ``[batch, seq, heads, dim]``; ``prev_kv[i - 1]`` is the stacked
+    ``[2, batch, seq, kv_heads, dim]`` chunk of rank ``rank - i``."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, window_size, cp_size, rank, softmax_scale, ring_dtypes, *prev_kv):
+        b, s, hq, d = q.shape
+        if softmax_scale is None:
+            softmax_scale = d ** (-0.5)
+        plan = plan_nonvarlen(s, window_size, cp_size, rank)
+        for (i, _, _, _, _) in plan:
+            assert i == 0 or i <= len(prev_kv), f"step {i} needs the chunk of rank {rank - i}"
+        out, lse = _forward_blocks(q, k, v, prev_kv, plan, softmax_scale, None, ring_dtypes)
+        ctx.save_for_backward(q, k, v, out, lse, *prev_kv)
+        ctx.plan, ctx.scale = plan, softmax_scale
+        return out
+
+    @staticmethod
+    def backward(ctx, do):
+        q, k, v, out, lse, *prev_kv = ctx.saved_tensors
+        grads = _backward_blocks(q, k, v, prev_kv, out, lse, do, ctx.plan, ctx.scale, None)
+        return (grads[0], grads[1], grads[2], None, None, None, None, None, *grads[3:])
+
+
+class RankShareVarlenFunc(torch.autograd.Function):
+    """Packed tensors ``[tokens, heads, dim]``; ``prev_kv[i - 1]`` is ``[2, tokens, kv_heads, dim]``."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, window_size, cu_host, cp_size, rank, softmax_scale, ring_dtypes,
+                *prev_kv):
+        s, hq, d = q.shape
+        if softmax_scale is None:
+            softmax_scale = d ** (-0.5)
+        local_cu, plan = plan_varlen(cu_host, s, window_size, cp_size, rank)
+        cu_dev = torch.tensor(local_cu, dtype=torch.int32, device=q.device)
+        q4, k4, v4 = q.unsqueeze(0), k.unsqueeze(0), v.unsqueeze(0)
+        prev4 = [p.unsqueeze(1) for p in prev_kv]
+        out, lse = _forward_blocks(q4, k4, v4, prev4, plan, softmax_scale, cu_dev, ring_dtypes)
+        out, lse = out.squeeze(0), lse.squeeze(0)
+        ctx.save_for_backward(q, k, v, out, lse, cu_dev, *prev_kv)
+        ctx.plan, ctx.scale = plan, softmax_scale
+        return out
+
+    @staticmethod
+    def backward(ctx, do):
+        q, k, v, out, lse, cu_dev, *prev_kv = ctx.saved_tensors
+        prev4 = [p.unsqueeze(1) for p in prev_kv]
+        grads = _backward_blocks(q.unsqueeze(0), k.unsqueeze(0), v.unsqueeze(0), prev4,
+                                 out.unsqueeze(0), lse.unsqueeze(0), do.unsqueeze(0), ctx.plan,
+                                 ctx.scale, cu_dev)
+        dprev = [g.squeeze(1) for g in grads[3:]]
+        return (grads[0].squeeze(0), grads[1].squeeze(0), grads[2].squeeze(0), None, None, None,
+                None, None, None, *dprev)
+
+
+def _forward_blocks(q, k, v, prev_kv, plan, scale, local_cu, ring_dtypes):
+    """Run the planned blocks and merge them.  Dense 4-d tensors (batch 1 when packed)."""
+    b, s, hq, d = q.shape
+    out = lse = None
+    for (i, qs, ks, window, causal) in plan:
+        kk, vv = (k, v) if i == 0 else (prev_kv[i - 1][0], prev_kv[i - 1][1])
+        if i == 0 and local_cu is not None:
+            o_i, l_i = attn_fwd(q[0], kk[0], vv[0], scale, window, causal, local_cu, local_cu)
+            o_i, l_i = o_i.unsqueeze(0), l_i.unsqueeze(0)
+        else:
+            o_i, l_i = attn_fwd(q[:, qs], kk[:, ks], vv[:, ks], scale, window, causal)
+        if out is None:
+            # the diagonal block covers every row: it seeds the accumulators directly
+            assert i == 0
+            if ring_dtypes:
+                # accumulator types of ring_swa/sliding_window/nonvarlen.py:53-59
+                out, lse = o_i.float(), l_i.double()
+            else:
+                out, lse = o_i, l_i
+        else:
+            merge_attn_out(out[:, qs], lse[:, :, qs], o_i, l_i)
+    return out.to(q.dtype), lse.float()
+
+
+def _backward_blocks(q, k, v, prev_kv, out, lse, do, plan, scale, local_cu):
+    if do.stride(-1) != 1:
+        do = do.contiguous()
+    single = len(plan) == 1
+    dq_acc = None if single else torch.zeros_like(q, dtype=torch.float32)
+    dq = dk = dv = None
+    dprev = [None] * len(prev_kv)
+    for (i, qs, ks, window, causal) in plan:
+        kk, vv = (k, v) if i == 0 else (prev_kv[i - 1][0], prev_kv[i - 1][1])
+        if i == 0:
+            dq_i, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+            if local_cu is not None:
+                attn_bwd(q[0], kk[0], vv[0], out[0], lse[0], do[0], dq_i[0], dk[0], dv[0], scale,
+                         window, causal, local_cu, local_cu)
+            else:
+                attn_bwd(q, kk, vv, out, lse, do, dq_i, dk, dv, scale, window, causal)
+            if single:
+                dq = dq_i
+            else:
+                dq_acc.add_(dq_i)
+        else:
+            # rows / keys outside the slices receive nothing from this block
+            dkv = torch.zeros_like(prev_kv[i - 1])
+            dq_i = torch.empty_like(q[:, qs])
+            attn_bwd(q[:, qs], kk[:, ks], vv[:, ks], out[:, qs], lse[:, :, qs], do[:, qs], dq_i,
+                     dkv[0][:, ks], dkv[1][:, ks], scale, window, causal)
+            dq_acc[:, qs].add_(dq_i)
+            dprev[i - 1] = dkv
+    if not single:
+        dq = dq_acc.to(q.dtype)
+    for n, g in enumerate(dprev):
+        if g is None:
+            dprev[n] = torch.zeros_like(prev_kv[n])
+    return (dq, dk, dv, *dprev)
+
+
+def ring_rank_share_attn(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    prev_kv: Sequence[torch.Tensor],
+    window_size: int,
+    cp_size: int,
+    cp_local_rank: int,
+    softmax_scale: Optional[float] = None,
+    *,
+    ring_dtypes: bool = False,
+) -> torch.Tensor:
+    """Attention output of rank ``cp_local_rank`` for its chunk ``q, k, v``
+    (``[batch, seq, heads, dim]``), given ``prev_kv[i - 1] = stack([k, v])`` of rank
+    ``cp_local_rank - i``.  Differentiable w.r.t. ``q, k, v`` and every ``prev_kv``
+    entry (the gradient a real ring would send back).  ``ring_dtypes=True`` keeps the
+    running output in fp32 and the running LSE in fp64 as upstream does."""
+    assert q.shape[1] == k.shape[1] == v.shape[1], "Sequence length must be the same"
+    return RankShareFunc.apply(q, k, v, int(window_size), int(cp_size), int(cp_local_rank),
+                               softmax_scale, bool(ring_dtypes), *prev_kv)
+
+
+def ring_rank_share_attn_varlen(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    prev_kv: Sequence[torch.Tensor],
+    window_size: int,
+    cu_seqlens,
+    cp_size: int,
+    cp_local_rank: int,
+    softmax_scale: Optional[float] = None,
+    *,
+    ring_dtypes: bool = False,
+) -> torch.Tensor:
+    """Packed twin: ``q, k, v`` are the rank's ``[tokens, heads, dim]`` slice of the
+    pack and ``cu_seqlens`` the cumulative lengths of the WHOLE pack (a host list or a
+    tensor, read once on the host to lay out the blocks)."""
+    cu_host = cu_seqlens.tolist() if torch.is_tensor(cu_seqlens) else list(cu_seqlens)
+    assert q.shape[0] == cu_host[-1] // cp_size, (
+        "cu_seqlens does not match with sequence length per rank"
+    )
+    return RankShareVarlenFunc.apply(q, k, v, int(window_size), cu_host, int(cp_size),
+                                     int(cp_local_rank), softmax_scale, bool(ring_dtypes), *prev_kv)
