@@ -1,0 +1,257 @@
+"""Benchmark of the single-GPU attention path on one MI355X.
+
+Headline workload (``config.workload = "c3_rank_share"``): one context-parallel
+rank's share of ring sliding-window attention — bf16, batch 1, local chunk 8192
+tokens of a 65536-token sequence (virtual cp 8), 32 q / 8 kv heads, head_dim
+128, window 4096: band attention on the rank's own chunk, the upper-right
+4096 x 4096 corner against the previous rank's chunk held in HBM, LSE merge of
+the two partials; forward + backward through autograd.  One "step" = one such
+forward + backward.  ``value`` = window-effective TFLOP/s =
+14 * D * pairs * Hq / time with pairs = 8192 * 4097 unmasked (query, key) pairs
+per head.  Inputs are synthetic N(0,1), seeded, resident in HBM before timing.
+
+Prints ONE JSON line.  ``python bench.py`` defaults to 1 GPU and finishes in
+about a minute; ``--gpus N`` with N > 1 is refused (this build is single-GPU).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_HBM_GBPS = 8000.0     # MI355X HBM3E
+
+
+def band_pairs(length: int, w: int) -> int:
+    return length * (length + 1) // 2 if length <= w + 1 else (w + 1) * length - w * (w + 1) // 2
+
+
+def event_ms(fn, n, warm=3):
+    """Median duration of fn() on torch's current stream (the stream the C ABI launches
+    on), measured with HIP events."""
+    import torch
+
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    evs = [torch.cuda.Event(enable_timing=True) for _ in range(n + 1)]
+    evs[0].record()
+    for i in range(n):
+        fn()
+        evs[i + 1].record()
+    torch.cuda.synchronize()
+    ts = sorted(evs[i].elapsed_time(evs[i + 1]) for i in range(n))
+    return ts[len(ts) // 2], sum(ts) / len(ts)
+
+
+def cpu_baseline(seconds_budget: float = 25.0):
+    """The oracle (PyTorch masked softmax, fp32, autograd) on the host cores.
+
+    Bounded sample of the headline workload: same structure scaled down — chunk 4096
+    with a 4096-token predecessor, window 2048, 4 q / 1 kv heads, head_dim 128 — plus
+    the reference's own CPU-runnable case (fp32, seq 1024, 4 heads, head_dim 64,
+    window 256, seed 0)."""
+    import torch
+
+    from oracle import attention_oracle as O
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+
+    def run(sq, sk, hq, hk, d, w, seed):
+        g = torch.Generator().manual_seed(seed)
+        q = torch.randn(1, sq, hq, d, generator=g)
+        k = torch.randn(1, sk, hk, d, generator=g)
+        v = torch.randn(1, sk, hk, d, generator=g)
+        do = torch.randn(1, sq, hq, d, generator=g)
+        fn = lambda: O.attention_fwd_bwd(  # noqa: E731
+            lambda q, k, v: O.window_attention(q, k, v, d ** -0.5, (w, 0), True), q, k, v, do)
+        fn()
+        ts = []
+        t_start = time.perf_counter()
+        while len(ts) < 5 and (time.perf_counter() - t_start < seconds_budget / 2 or len(ts) < 2):
+            t0 = time.perf_counter()
+            fn()
+            ts.append(time.perf_counter() - t0)
+        ts.sort()
+        return ts[len(ts) // 2]
+
+    # sample of the rank share: queries = last 4096 positions of 8192 keys, window 2048
+    sq, sk, hq, hk, d, w = 4096, 8192, 4, 1, 128, 2048
+    t = run(sq, sk, hq, hk, d, w, 0)
+    pairs = sq * (w + 1)  # every query has a full window inside the two chunks
+    sample_tflops = 14 * d * pairs * hq / t / 1e12
+    t1 = run(1024, 1024, 4, 4, 64, 256, 0)
+    c1_gflops = 14 * 64 * band_pairs(1024, 256) * 4 / t1 / 1e9
+    return {
+        "value": sample_tflops,
+        "unit": "TFLOP/s",
+        "cores": cores,
+        "threads": torch.get_num_threads(),
+        "kind": "port",
+        "sample": "oracle fp32 fwd+bwd (autograd) of a scaled-down rank share: 4096 queries x "
+                  "8192 keys (own + previous chunk), window 2048, 4 q / 1 kv heads, head_dim 128; "
+                  f"median {t * 1e3:.1f} ms",
+        "c1_fp32_seq1024_h4_d64_w256": {"ms": t1 * 1e3, "GFLOP/s": c1_gflops},
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true", help="skip the per-kernel / merge extras")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this build covers the single-GPU path only; run with --gpus 1 "
+                 "(one rank's share of the ring is emulated on that GPU)")
+
+    import __graft_entry__ as entry
+
+    entry.ensure_built()
+    import torch
+
+    import ring_swa
+    from ring_swa.ops import attn_bwd, attn_fwd, merge_attn_out
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    torch.manual_seed(0)
+
+    # ---- headline workload ------------------------------------------------------
+    S, HQ, HK, D, W, CP, RANK = 8192, 32, 8, 128, 4096, 8, 1
+    mk = lambda *shape: torch.randn(*shape, device=dev, dtype=torch.bfloat16)  # noqa: E731
+    q, k, v = mk(1, S, HQ, D).requires_grad_(), mk(1, S, HK, D).requires_grad_(), \
+        mk(1, S, HK, D).requires_grad_()
+    prev = mk(2, 1, S, HK, D).requires_grad_()
+    do = mk(1, S, HQ, D)
+    pairs_diag = band_pairs(S, W)
+    pairs_off = W * (W + 1) // 2
+    pairs = pairs_diag + pairs_off
+    assert pairs == S * (W + 1)
+    flops = 14 * D * pairs * HQ
+
+    def step():
+        for t in (q, k, v, prev):
+            t.grad = None
+        out = ring_swa.ring_rank_share_attn(q, k, v, [prev], W, CP, RANK)
+        out.backward(do)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    value = flops / (ms * 1e-3) / 1e12
+
+    rec = {
+        "metric": "fwd+bwd window-effective TFLOP/s + % bf16 MFMA peak; merge GB/s, 1 MI355X",
+        "value": value,
+        "unit": "TFLOP/s",
+        "pct_bf16_mfma_peak": 100.0 * value / PEAK_BF16_TFLOPS,
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": "c3_rank_share",
+            "detail": "1 rank of virtual cp 8: chunk 8192 of seq 65536, 32 q / 8 kv heads, "
+                      "head_dim 128, window 4096; own-chunk band + previous-chunk corner + LSE "
+                      "merge; fwd+bwd via autograd",
+            "batch": 1, "chunk": S, "heads_q": HQ, "heads_kv": HK, "head_dim": D, "window": W,
+            "pairs_per_head": pairs, "flops_per_step": flops,
+        },
+    }
+
+    # ---- roofline of the dominant kernel: backward main kernel, own-chunk block ----
+    with torch.no_grad():
+        qd, kd, vd = q.detach(), k.detach(), v.detach()
+        o_d, lse_d = attn_fwd(qd, kd, vd, None, (W, 0), True)
+        dq, dk, dv = torch.empty_like(qd), torch.empty_like(kd), torch.empty_like(vd)
+        from ring_swa import _lib
+        ws = torch.empty(int(64 + qd.numel() * 4 + qd.numel() // D * 4 + 4096), dtype=torch.uint8,
+                         device=dev)
+        bwd = lambda ph: attn_bwd(qd, kd, vd, o_d, lse_d, do, dq, dk, dv, None, (W, 0), True,  # noqa: E731
+                                  workspace=ws, phases=ph)
+        bwd(7)
+        n = 5 if args.no_extras else 20
+        main_med, main_avg = event_ms(lambda: bwd(2), n)
+        fl_main = 10 * D * pairs_diag * HQ
+        rec["roofline"] = {
+            "kernel": "attn_bwd_kernel<bf16,128> (own-chunk block 8192x8192, window 4096)",
+            "bound": "mfma",
+            "achieved": fl_main / (main_avg * 1e-3) / 1e12,
+            "peak": PEAK_BF16_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": fl_main / (main_avg * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+            "traffic": None,
+            "avg_launch_ms": main_avg,
+            "median_launch_ms": main_med,
+            "flops_per_launch": fl_main,
+        }
+        if not args.no_extras:
+            fwd_med, _ = event_ms(lambda: attn_fwd(qd, kd, vd, None, (W, 0), True), 20)
+            bwd_med, _ = event_ms(lambda: bwd(7), 20)
+            fl_fwd = 4 * D * pairs_diag * HQ
+            rec["kernels"] = {
+                "fwd_own_chunk": {"ms": fwd_med, "TFLOP/s": fl_fwd / fwd_med / 1e9},
+                "bwd_own_chunk_all_phases": {"ms": bwd_med, "TFLOP/s": fl_main / bwd_med / 1e9},
+                "bwd_own_chunk_main_kernel": {"ms": main_med, "TFLOP/s": fl_main / main_med / 1e9},
+            }
+            # config 2: plain single-GPU SWA, batch 2, seq 8192, 32/32 heads, window 1000
+            q2, k2, v2, do2 = (mk(2, 8192, 32, 128) for _ in range(4))
+            o2, l2 = attn_fwd(q2, k2, v2, None, (1000, 0), True)
+            g2 = [torch.empty_like(q2) for _ in range(3)]
+            f2, _ = event_ms(lambda: attn_fwd(q2, k2, v2, None, (1000, 0), True), 10)
+            b2, _ = event_ms(lambda: attn_bwd(q2, k2, v2, o2, l2, do2, *g2, None, (1000, 0), True), 10)
+            p2 = band_pairs(8192, 1000) * 2 * 32
+            rec["c2_swa_b2_s8192_h32_w1000"] = {
+                "fwd_ms": f2, "bwd_ms": b2, "TFLOP/s": 14 * 128 * p2 / (f2 + b2) / 1e9,
+                "pct_bf16_mfma_peak": 14 * 128 * p2 / (f2 + b2) / 1e9 / PEAK_BF16_TFLOPS * 100}
+            del q2, k2, v2, do2, o2, l2, g2
+            # merge kernel: rank-share shape (rows [:4096] x 32 heads) and the sweep's top point
+            merges = {}
+            for name, rows_s in (("c3_rows4096", 4096), ("sweep_s131072", 131072)):
+                acc = torch.randn(1, rows_s, HQ, D, device=dev)
+                lacc = torch.randn(1, HQ, rows_s, device=dev, dtype=torch.float64)
+                new = torch.randn(1, rows_s, HQ, D, device=dev, dtype=torch.bfloat16)
+                lnew = torch.randn(1, HQ, rows_s, device=dev)
+                med, avg = event_ms(lambda: merge_attn_out(acc, lacc, new, lnew), 20)
+                nbytes = rows_s * HQ * (10 * D + 20)
+                merges[name] = {"rows": rows_s * HQ, "bytes": nbytes, "us": med * 1e3,
+                                "GB/s": nbytes / med / 1e6,
+                                "dtypes": "o fp32, new o bf16, lse fp64, new lse fp32"}
+                if name == "sweep_s131072":
+                    rec["roofline_merge"] = {
+                        "kernel": "merge_kernel<float,bf16,16>", "bound": "hbm",
+                        "achieved": nbytes / avg / 1e6, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                        "frac": nbytes / avg / 1e6 / PEAK_HBM_GBPS, "traffic": None,
+                        "avg_launch_ms": avg, "bytes_per_launch": nbytes}
+                del acc, lacc, new, lnew
+            rec["merge"] = merges
+            rec["merge_GBps"] = merges["sweep_s131072"]["GB/s"]
+
+    if not args.no_cpu_baseline:
+        rec["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(rec))
+
+
+if __name__ == "__main__":
+    main()

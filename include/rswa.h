@@ -160,6 +160,19 @@ typedef struct rswa_attn_params {
 int rswa_attn_fwd(const rswa_attn_params* p, void* stream);
 int rswa_attn_bwd(const rswa_attn_params* p, void* stream);
 
+/*
+ * rswa_attn_bwd is three launches: PREP (delta = rowsum(dout * out), zero the fp32
+ * dq accumulator in the workspace), MAIN (dk, dv written; dq accumulated in the
+ * workspace) and POST (dq = cast(scale * accumulator)).  This variant enqueues only
+ * the phases named in the bit mask, on the same workspace: it lets a profiler or
+ * benchmark bracket the main kernel alone.  Same interface replaced as rswa_attn_bwd
+ * (ring_swa/ops/wrap_flash.py:276-429).
+ */
+#define RSWA_BWD_PREP 1
+#define RSWA_BWD_MAIN 2
+#define RSWA_BWD_POST 4
+int rswa_attn_bwd_phases(const rswa_attn_params* p, void* stream, int phases);
+
 /* Scratch rswa_attn_bwd needs for these shapes (fp32 dq accumulator + row sums). */
 uint64_t rswa_attn_bwd_workspace_bytes(const rswa_attn_params* p);
 

@@ -442,11 +442,11 @@ __global__ __launch_bounds__(256) void attn_bwd_post_kernel(const AttnArgs a) {
 }
 
 template <typename T, int D>
-int launch_bwd(AttnArgs& a, hipStream_t stream) {
+int launch_bwd(AttnArgs& a, hipStream_t stream, int phases) {
   using C = BwdCfg<D>;
   const int64_t units = a.rows_q * a.heads_q;
   const unsigned ew_blocks = (unsigned)ceil_div(units * (D / 8), 256);
-  if (units > 0) {
+  if (units > 0 && (phases & RSWA_BWD_PREP)) {
     hipLaunchKernelGGL((attn_bwd_prep_kernel<T, D>), dim3(ew_blocks), dim3(256), 0, stream, a);
     int rc = check_launch("attn_bwd prep");
     if (rc != RSWA_OK) return rc;
@@ -458,7 +458,7 @@ int launch_bwd(AttnArgs& a, hipStream_t stream) {
     a.n_tile = (int)ceil_div(a.seqlen_k, C::BN);
     a.n_work = a.n_tile * a.heads_kv * a.batch;
   }
-  if (a.n_work > 0) {
+  if (a.n_work > 0 && (phases & RSWA_BWD_MAIN)) {
     auto kern = attn_bwd_kernel<T, D>;
     static bool configured = false;  // benign race: the attribute call is idempotent
     if (!configured) {
@@ -472,28 +472,30 @@ int launch_bwd(AttnArgs& a, hipStream_t stream) {
     int rc = check_launch("attn_bwd main");
     if (rc != RSWA_OK) return rc;
   }
-  if (units > 0) {
+  if (units > 0 && (phases & RSWA_BWD_POST)) {
     hipLaunchKernelGGL((attn_bwd_post_kernel<T, D>), dim3(ew_blocks), dim3(256), 0, stream, a);
     return check_launch("attn_bwd post");
   }
   return RSWA_OK;
 }
 
-// dk / dv rows no block owns (none today: every key row belongs to exactly one block
-// that always writes it), kept explicit for the reader: blocks with no visible query
-// still write zeros because their accumulators start at zero.
-
 }  // namespace
 }  // namespace rswa
 
-extern "C" int rswa_attn_bwd(const rswa_attn_params* p, void* stream) {
+extern "C" int rswa_attn_bwd_phases(const rswa_attn_params* p, void* stream, int phases) {
   using namespace rswa;
   AttnArgs a;
   int rc = fill_args(p, true, a);
   if (rc != RSWA_OK) return rc;
   hipStream_t st = (hipStream_t)stream;
   if (p->dtype == RSWA_BF16) {
-    return p->head_dim == 128 ? launch_bwd<__bf16, 128>(a, st) : launch_bwd<__bf16, 64>(a, st);
+    return p->head_dim == 128 ? launch_bwd<__bf16, 128>(a, st, phases)
+                              : launch_bwd<__bf16, 64>(a, st, phases);
   }
-  return p->head_dim == 128 ? launch_bwd<_Float16, 128>(a, st) : launch_bwd<_Float16, 64>(a, st);
+  return p->head_dim == 128 ? launch_bwd<_Float16, 128>(a, st, phases)
+                            : launch_bwd<_Float16, 64>(a, st, phases);
+}
+
+extern "C" int rswa_attn_bwd(const rswa_attn_params* p, void* stream) {
+  return rswa_attn_bwd_phases(p, stream, RSWA_BWD_PREP | RSWA_BWD_MAIN | RSWA_BWD_POST);
 }

@@ -106,6 +106,8 @@ def lib() -> ctypes.CDLL:
         fn = getattr(L, name)
         fn.restype = c_int
         fn.argtypes = [POINTER(AttnParams), c_void_p]
+    L.rswa_attn_bwd_phases.restype = c_int
+    L.rswa_attn_bwd_phases.argtypes = [POINTER(AttnParams), c_void_p, c_int]
     L.rswa_attn_bwd_workspace_bytes.restype = c_uint64
     L.rswa_attn_bwd_workspace_bytes.argtypes = [POINTER(AttnParams)]
     if L.rswa_sizeof_attn_params() != ctypes.sizeof(AttnParams):

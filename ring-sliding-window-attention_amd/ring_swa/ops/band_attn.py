@@ -141,8 +141,14 @@ def attn_bwd(
     *,
     num_sink: int = 0,
     mask_shift: Optional[int] = None,
+    workspace: Optional[torch.Tensor] = None,
+    phases: int = 7,
 ) -> None:
-    """Masked attention backward; overwrites ``dq, dk, dv`` (views are fine)."""
+    """Masked attention backward; overwrites ``dq, dk, dv`` (views are fine).
+
+    ``workspace`` (uint8, at least ``rswa_attn_bwd_workspace_bytes``) may be supplied to
+    avoid the per-call scratch allocation; ``phases`` is the bit mask of
+    ``rswa_attn_bwd_phases`` (1 prep, 2 main, 4 post) for profiling."""
     packed = cu_seqlens_q is not None
     _check_qkv(q, k, v, packed)
     dev = _lib.require_device(q, k, v, o, softmax_lse, do, dq, dk, dv)
@@ -180,11 +186,13 @@ def attn_bwd(
     p.dv_stride = _lib.i64x3(_strides3(dv, packed))
     L = _lib.lib()
     need = int(L.rswa_attn_bwd_workspace_bytes(p))
-    ws = torch.empty(need, dtype=torch.uint8, device=dev)  # caching allocator: 512-B aligned
-    p.workspace = ws.data_ptr()
-    p.workspace_bytes = need
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=dev)  # 512-B aligned by torch
+    assert workspace.dtype == torch.uint8 and workspace.numel() >= need and workspace.device == dev
+    p.workspace = workspace.data_ptr()
+    p.workspace_bytes = workspace.numel()
     with torch.cuda.device(dev):
-        _lib.check(L.rswa_attn_bwd(p, _lib.stream_ptr(dev)))
+        _lib.check(L.rswa_attn_bwd_phases(p, _lib.stream_ptr(dev), int(phases)))
 
 
 # ---- names of the upstream wrappers -----------------------------------------
