@@ -180,7 +180,7 @@ def main():
         },
     }
 
-    # ---- roofline of the dominant kernel: backward main kernel, own-chunk block ----
+    # ---- roofline of the dominant kernel: backward dK/dV kernel, own-chunk block ----
     with torch.no_grad():
         qd, kd, vd = q.detach(), k.detach(), v.detach()
         o_d, lse_d = attn_fwd(qd, kd, vd, None, (W, 0), True)

@@ -106,10 +106,9 @@ int rswa_merge_attn_out(void* o, int o_dtype, const int64_t* o_stride,
  * several blocks, which is how the ring's "merge backward" is realised
  * (ring_swa/sliding_window/nonvarlen.py:242-253) — and OVERWRITES dq, dk, dv
  * (rows/keys that receive nothing are written as zero).  dk/dv are reduced over
- * the heads_q / heads_kv query heads that share a kv head.  dq is accumulated
- * with fp32 atomics in `workspace`, so its low-order bits are not run-to-run
- * deterministic (upstream flash-attn runs with deterministic=False as well,
- * ring_swa/ops/wrap_flash.py:61).
+ * the heads_q / heads_kv query heads that share a kv head.  No atomics are used:
+ * results are run-to-run deterministic (upstream runs flash-attn with
+ * deterministic=False, ring_swa/ops/wrap_flash.py:61).
  */
 typedef struct rswa_attn_params {
   int32_t dtype;    /* RSWA_BF16 or RSWA_F16: type of q,k,v,out,dout,dq,dk,dv */
@@ -161,19 +160,19 @@ int rswa_attn_fwd(const rswa_attn_params* p, void* stream);
 int rswa_attn_bwd(const rswa_attn_params* p, void* stream);
 
 /*
- * rswa_attn_bwd is three launches: PREP (delta = rowsum(dout * out), zero the fp32
- * dq accumulator in the workspace), MAIN (dk, dv written; dq accumulated in the
- * workspace) and POST (dq = cast(scale * accumulator)).  This variant enqueues only
- * the phases named in the bit mask, on the same workspace: it lets a profiler or
- * benchmark bracket the main kernel alone.  Same interface replaced as rswa_attn_bwd
- * (ring_swa/ops/wrap_flash.py:276-429).
+ * rswa_attn_bwd is three launches: PREP (delta = rowsum(dout * out) into the
+ * workspace), DKDV (dk, dv written; reads delta) and DQ (dq written; reads delta).
+ * This variant enqueues only the phases named in the bit mask, on the same
+ * workspace: it lets a profiler or benchmark bracket one kernel alone, and lets a
+ * caller that needs only some of the gradients skip the rest.  Same interface
+ * replaced as rswa_attn_bwd (ring_swa/ops/wrap_flash.py:276-429).
  */
 #define RSWA_BWD_PREP 1
-#define RSWA_BWD_MAIN 2
-#define RSWA_BWD_POST 4
+#define RSWA_BWD_DKDV 2
+#define RSWA_BWD_DQ 4
 int rswa_attn_bwd_phases(const rswa_attn_params* p, void* stream, int phases);
 
-/* Scratch rswa_attn_bwd needs for these shapes (fp32 dq accumulator + row sums). */
+/* Scratch rswa_attn_bwd needs for these shapes (fp32 row sums of dout * out). */
 uint64_t rswa_attn_bwd_workspace_bytes(const rswa_attn_params* p);
 
 /* Message of the calling thread's last failed call ("" if none). */

@@ -5,12 +5,6 @@ namespace rswa {
 
 static uint64_t align_up(uint64_t x, uint64_t a) { return (x + a - 1) / a * a; }
 
-static uint64_t dq_acc_bytes(const rswa_attn_params* p) {
-  const uint64_t rows = p->cu_seqlens_q ? (uint64_t)p->total_q
-                                        : (uint64_t)p->batch * (uint64_t)p->seqlen_q;
-  return align_up(rows * (uint64_t)p->heads_q * (uint64_t)p->head_dim * sizeof(float), 256);
-}
-
 static uint64_t delta_bytes(const rswa_attn_params* p) {
   const uint64_t rows = p->cu_seqlens_q ? (uint64_t)p->total_q
                                         : (uint64_t)p->batch * (uint64_t)p->seqlen_q;
@@ -19,7 +13,7 @@ static uint64_t delta_bytes(const rswa_attn_params* p) {
 
 uint64_t bwd_workspace_bytes(const rswa_attn_params* p) {
   if (!p || p->batch <= 0 || p->heads_q <= 0 || p->head_dim <= 0) return 0;
-  return dq_acc_bytes(p) + delta_bytes(p);
+  return delta_bytes(p);
 }
 
 static bool rows_aligned(const void* ptr, const int64_t* st) {
@@ -66,7 +60,6 @@ int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a) {
   a.dq = p->dq;
   a.dk = p->dk;
   a.dv = p->dv;
-  a.dq_acc = nullptr;
   a.delta = nullptr;
   a.cu_q = p->cu_seqlens_q;
   a.cu_k = p->cu_seqlens_k;
@@ -116,8 +109,7 @@ int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a) {
                  (unsigned long long)p->workspace_bytes, (unsigned long long)need);
     RSWA_REQUIRE(((uintptr_t)p->workspace) % 256 == 0, RSWA_ERR_INVALID,
                  "attn_bwd: workspace must be 256-byte aligned");
-    a.dq_acc = (float*)p->workspace;
-    a.delta = (float*)((char*)p->workspace + dq_acc_bytes(p));
+    a.delta = (float*)p->workspace;
   }
   return RSWA_OK;
 }

@@ -1,69 +1,70 @@
-// Band / sink attention backward for gfx950.
+// Band / sink attention backward for gfx950, without atomics.
 //
 // Replaces flash-attn's backward as wrapped at ring_swa/ops/wrap_flash.py:276-429.
 // Three launches on the caller's stream:
-//   1. prep : delta[h][row] = sum_d dO*O (fp32) and zero of the fp32 dQ accumulator
-//   2. main : one block owns 128 keys of one (sequence, kv head) and walks the query
-//             tiles (64 rows) that can see them, for every q head of the GQA group;
-//             dK^T / dV^T stay in registers for the whole walk, dQ goes out through
-//             fp32 atomics
-//   3. post : dq = cast(scale * dq_acc)
+//   PREP : delta[h][row] = sum_d dO * O   (fp32, in the caller's workspace)
+//   DKDV : one block owns 128 keys of one (sequence, kv head) and walks the query tiles
+//          (64 rows) that can see them, for every q head of the GQA group; dK^T / dV^T
+//          stay in registers for the whole walk and are written once
+//   DQ   : one block owns 128 queries of one (sequence, q head) and walks the key tiles
+//          (64 keys) it can see, like the forward kernel; dQ^T stays in registers
+// S and dP are computed in both main kernels (7 GEMM units instead of 5).  That costs
+// less here than fp32 atomics on dQ: the L2 retires about one fp32 atomic per clock per
+// channel, which caps an atomic dQ far below the MFMA rate.  It also makes the result
+// run-to-run deterministic.
 //
-// Main-kernel data flow per (query tile, wave); wave w owns key columns 32w..32w+31:
-//   S  = Q K^T, dP = dO V^T     A = Q / dO rows from LDS, B = K / V fragments (registers)
-//   P  = exp2(S*c - lse*log2e), dS = P * (dP - delta)           (C layout: lane = key)
-//   dV^T += dO^T P, dK^T += Q^T dS   A = transposing LDS reads of dO / Q, B = P / dS regs
-//   dS^T -> LDS; dQ[:, d-slice] = dS K   A = transposing reads of dS^T, B = K^T fragments
+// DKDV per (query tile, wave); wave w owns key columns 32w..32w+31 (C layout: lane = key):
+//   S = Q K^T, dP = dO V^T      A = Q / dO row fragments from LDS, B = K / V fragments (regs)
+//   P = exp2(S*c - lse*log2e), dS = P * (dP - delta)
+//   dV^T += dO^T P, dK^T += Q^T dS   A = transposing LDS reads of dO / Q, B = P / dS (regs)
+// DQ per (key tile, wave); wave w owns query columns 32w..32w+31 (C layout: lane = query):
+//   S^T = K Q^T, dP^T = V dO^T  A = K / V row fragments from LDS, B = Q / dO fragments (regs)
+//   dS^T as above with per-lane lse / delta
+//   dQ^T += K^T dS^T            A = transposing LDS reads of K, B = dS^T (regs)
 #include "attn_common.h"
 
 namespace rswa {
 namespace {
 
-// XOR swizzle of 16-byte chunks inside an LDS tile whose rows hold CH chunks (8 or 16).
-// It makes both access patterns used here bank-conflict free: 16 consecutive rows at one
-// logical chunk (MFMA row fragments, 16-byte reads) and 4 consecutive rows x 4 consecutive
-// chunks (one phase of the transposing 8-byte reads).
-template <int CH>
-__device__ __forceinline__ int swz(int row, int chunk) {
-  if constexpr (CH == 16) {
-    return chunk ^ (((row & 3) << 2) | ((row >> 2) & 3));
-  } else {
-    static_assert(CH == 8, "rows of 8 or 16 chunks");
-    return chunk ^ ((((row >> 1) & 1) << 2) | ((row >> 2) & 3));
-  }
+typedef __attribute__((__vector_size__(8 * sizeof(short)))) short s16x8;
+
+// Two transposing reads -> one 8-element MFMA fragment.
+template <typename V8>
+__device__ __forceinline__ V8 tr_pair(const char* p0, const char* p1) {
+  const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p0);
+  const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p1);
+  const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  V8 out;
+  __builtin_memcpy(&out, &both, 16);
+  return out;
 }
 
+// ============================================================================
+// dK / dV
+// ============================================================================
 template <int D>
-struct BwdCfg {
+struct DkvCfg {
   static constexpr int BM = 64;   // query rows per step
   static constexpr int BN = 128;  // keys per block
   static constexpr int THREADS = 256;
   static constexpr int MI = BM / 32;
   static constexpr int KSTEPS = D / 16;
   static constexpr int DBLK = D / 32;
-  static constexpr int CPR = D / 8;                      // chunks per row of a [*, D] tile
-  static constexpr int ROWB = D * 2;                     // bytes per row
-  static constexpr int QCH = BM * CPR / THREADS;         // chunks per thread per Q (or dO) tile
-  static constexpr int KCH = BN * CPR / THREADS;
-  static constexpr int DQ_TILES = MI * DBLK / 4;         // dQ 32x32 tiles per wave
+  static constexpr int CPR = D / 8;   // 16-byte chunks per row
+  static constexpr int ROWB = D * 2;  // bytes per row
+  static constexpr int QCH = BM * CPR / THREADS;
   static constexpr int Q_TILE = BM * ROWB;
-  static constexpr int DS_ROWB = BM * 2;                 // dS^T tile: [BN keys][BM queries]
-  static constexpr int DS_TILE = BN * DS_ROWB;
-  static constexpr int OFF_Q = 0;                        // 2 buffers
-  static constexpr int OFF_DO = 2 * Q_TILE;              // 2 buffers
-  static constexpr int OFF_DS = 4 * Q_TILE;
-  static constexpr int OFF_ST = OFF_DS + DS_TILE;        // lse2[2][BM], delta[2][BM] fp32
+  static constexpr int OFF_Q = 0;            // 2 buffers
+  static constexpr int OFF_DO = 2 * Q_TILE;  // 2 buffers
+  static constexpr int OFF_ST = 4 * Q_TILE;  // lse2[2][BM], delta[2][BM] fp32
   static constexpr int SMEM = OFF_ST + 4 * BM * 4;
-  static_assert(BN * ROWB <= OFF_DS, "K staging aliases the Q/dO buffers");
-  static_assert(BM == 64, "dS^T rows are 8 chunks");
 };
 
 template <typename T, int D>
-__global__ __launch_bounds__(256) void attn_bwd_kernel(const AttnArgs a) {
-  using C = BwdCfg<D>;
+__global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
+  using C = DkvCfg<D>;
   using M = Mma<T>;
   using V8 = typename M::V8;
-  typedef __attribute__((__vector_size__(8 * sizeof(short)))) short s16x8;
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
   const int wid = logical_block_id(a.n_work);
@@ -102,18 +103,19 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(const AttnArgs a) {
   const T* v_ptr = (const T*)a.v + b * a.v_st[0] + s.k_row0 * a.v_st[1] + hk * a.v_st[2];
   T* dk_ptr = (T*)a.dk + b * a.dk_st[0] + s.k_row0 * a.dk_st[1] + hk * a.dk_st[2];
   T* dv_ptr = (T*)a.dv + b * a.dv_st[0] + s.k_row0 * a.dv_st[1] + hk * a.dv_st[2];
-  // packed row index of this sequence's first query (for the workspace arrays)
   const int64_t ws_row0 = a.cu_q ? s.q_row0 : (int64_t)b * a.seqlen_q;
 
   // ---- query tiles that can see this key tile -------------------------------
-  int i_min = (a.wr >= 0) ? max(0, j0 - shift - a.wr) : 0;
-  int i_max = (a.wl >= 0 && j0 >= a.n_sink) ? min(len_q - 1, j_last - shift + a.wl) : len_q - 1;
+  const int i_min = (a.wr >= 0) ? max(0, j0 - shift - a.wr) : 0;
+  const int i_max =
+      (a.wl >= 0 && j0 >= a.n_sink) ? min(len_q - 1, j_last - shift + a.wl) : len_q - 1;
   const int qt_lo = i_min / C::BM;
   const int n_qt = (i_max >= i_min) ? i_max / C::BM - qt_lo + 1 : 0;
   const int n_iter = n_qt * a.group;
 
-  // ---- K / V fragments -------------------------------------------------------
-  const int jc = j0 + wave * 32 + l32;  // this lane's key column
+  // ---- K / V fragments (B operands), resident for the whole walk --------------
+  const int jw0 = j0 + wave * 32;  // first key column of this wave
+  const int jc = jw0 + l32;        // this lane's key column
   V8 kf[C::KSTEPS], vf[C::KSTEPS];
 #pragma unroll
   for (int ks = 0; ks < C::KSTEPS; ks++) {
@@ -124,34 +126,6 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(const AttnArgs a) {
       kf[ks] = V8{0, 0, 0, 0, 0, 0, 0, 0};
       vf[ks] = V8{0, 0, 0, 0, 0, 0, 0, 0};
     }
-  }
-  // K^T fragments for dQ = dS K: B operand, lane = d column of this wave's d-block,
-  // slots = 8 consecutive keys.  Staged through LDS for the transposing read.
-  const int dq_db = wave % C::DBLK;
-  V8 ktf[C::BN / 16];
-  if (n_iter > 0) {
-#pragma unroll
-    for (int n = 0; n < C::KCH; n++) {
-      const int c = tid + n * C::THREADS;
-      const int row = c / C::CPR, ch = c % C::CPR;
-      u32x4 val = u32x4{0, 0, 0, 0};
-      if (j0 + row < len_k) val = *(const u32x4*)(k_ptr + (int64_t)(j0 + row) * a.k_st[1] + ch * 8);
-      *(u32x4*)(smem + row * C::ROWB + swz<C::CPR>(row, ch) * 16) = val;
-    }
-    __syncthreads();
-#pragma unroll
-    for (int ks = 0; ks < C::BN / 16; ks++) {
-      const int row = ks * 16 + 8 * g + (i16 >> 2);
-      const int ch = 4 * dq_db + 2 * (u & 1) + ((i16 & 3) >> 1);
-      const int half = (i16 & 1) * 8;
-      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-          (lds_s16x4*)(smem + row * C::ROWB + swz<C::CPR>(row, ch) * 16 + half));
-      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-          (lds_s16x4*)(smem + (row + 4) * C::ROWB + swz<C::CPR>(row + 4, ch) * 16 + half));
-      const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-      __builtin_memcpy(&ktf[ks], &both, 16);
-    }
-    __syncthreads();
   }
 
   f32x16 dk_acc[C::DBLK], dv_acc[C::DBLK];
@@ -229,139 +203,82 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(const AttnArgs a) {
     const float* lse_lds = (const float*)(smem + C::OFF_ST + buf * 2 * C::BM * 4);
     const float* delta_lds = lse_lds + C::BM;
 
-    // ---- S = Q K^T and dP = dO V^T (rows = queries, lane = key column) ------
-    f32x16 sacc[C::MI], pacc[C::MI];
-#pragma unroll
-    for (int mi = 0; mi < C::MI; mi++)
-#pragma unroll
-      for (int i = 0; i < 16; i++) {
-        sacc[mi][i] = 0.f;
-        pacc[mi][i] = 0.f;
-      }
-#pragma unroll
-    for (int ks = 0; ks < C::KSTEPS; ks++) {
-#pragma unroll
-      for (int mi = 0; mi < C::MI; mi++) {
-        const int row = mi * 32 + l32;
-        const int off = row * C::ROWB + swz<C::CPR>(row, ks * 2 + g) * 16;
-        const V8 qa = *(const V8*)(q_lds + off);
-        const V8 da = *(const V8*)(do_lds + off);
-        sacc[mi] = M::mfma32(qa, kf[ks], sacc[mi]);
-        pacc[mi] = M::mfma32(da, vf[ks], pacc[mi]);
-      }
-    }
-
-    // ---- P and dS -----------------------------------------------------------
-    // tile fully visible?  (every row valid, every key inside every row's band)
-    const int i_end = i0 + C::BM - 1;
-    const bool full = i_end < len_q && j0 + C::BN - 1 < len_k &&
-                      (a.wr < 0 || j0 + C::BN - 1 <= i0 + shift + a.wr) &&
-                      (a.wl < 0 || j0 >= i_end + shift - a.wl || j0 + C::BN - 1 < a.n_sink);
-#pragma unroll
-    for (int mi = 0; mi < C::MI; mi++) {
-#pragma unroll
-      for (int i4 = 0; i4 < 4; i4++) {
-        const int rbase = mi * 32 + 8 * i4 + 4 * g;
-        const f32x4 l4 = *(const f32x4*)(lse_lds + rbase);
-        const f32x4 d4 = *(const f32x4*)(delta_lds + rbase);
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-          const int i = 4 * i4 + e;
-          float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[mi][i], a.scale_log2, -l4[e]));
-          if (!full) {
-            const int iq = i0 + rbase + e;
-            const int rel = jc - iq - shift;  // key position relative to the aligned diagonal
-            const bool ok = jc < len_k && (a.wr < 0 || rel <= a.wr) &&
-                            (a.wl < 0 || rel >= -a.wl || jc < a.n_sink);
-            p = ok ? p : 0.f;  // invalid rows already have lse = +inf
-          }
-          sacc[mi][i] = p;
-          pacc[mi][i] = p * (pacc[mi][i] - d4[e]);
-        }
-      }
-    }
-
-    // ---- dV^T += dO^T P ; dK^T += Q^T dS --------------------------------------
-#pragma unroll
-    for (int ks = 0; ks < C::BM / 16; ks++) {
-      const int mi = ks >> 1;
-      float pv[8], dsv[8];
-#pragma unroll
-      for (int j = 0; j < 8; j++) {
-        pv[j] = sacc[mi][8 * (ks & 1) + j];
-        dsv[j] = pacc[mi][8 * (ks & 1) + j];
-      }
-      const V8 pb = M::pack(pv);
-      const V8 dsb = M::pack(dsv);
-      const int row = ks * 16 + 4 * g + (i16 >> 2);
-#pragma unroll
-      for (int d = 0; d < C::DBLK; d++) {
-        const int ch = 4 * d + 2 * (u & 1) + ((i16 & 3) >> 1);
-        const int half = (i16 & 1) * 8;
-        const int off0 = row * C::ROWB + swz<C::CPR>(row, ch) * 16 + half;
-        const int off1 = (row + 8) * C::ROWB + swz<C::CPR>(row + 8, ch) * 16 + half;
-        {
-          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(do_lds + off0));
-          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(do_lds + off1));
-          const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-          V8 af;
-          __builtin_memcpy(&af, &both, 16);
-          dv_acc[d] = M::mfma32(af, pb, dv_acc[d]);
-        }
-        {
-          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(q_lds + off0));
-          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(q_lds + off1));
-          const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-          V8 af;
-          __builtin_memcpy(&af, &both, 16);
-          dk_acc[d] = M::mfma32(af, dsb, dk_acc[d]);
-        }
-      }
-    }
-
-    // ---- dS^T -> LDS ([key][query], 8 chunks per row) --------------------------
-    {
-      char* ds_lds = smem + C::OFF_DS;
-      const int row = wave * 32 + l32;
+    // Does any (query of the tile, key of this wave) pair survive the mask?
+    const int i_end = min(i0 + C::BM, len_q) - 1;
+    const int jw1 = jw0 + 31;
+    const bool needed = jw0 < len_k && (a.wr < 0 || jw0 <= i_end + shift + a.wr) &&
+                        (a.wl < 0 || jw1 >= i0 + shift - a.wl || jw0 < a.n_sink);
+    if (needed) {
+      // ---- S = Q K^T and dP = dO V^T (rows = queries, lane = key column) ------
+      f32x16 sacc[C::MI], pacc[C::MI];
 #pragma unroll
       for (int mi = 0; mi < C::MI; mi++)
 #pragma unroll
-        for (int i4 = 0; i4 < 4; i4++) {
-          const auto h4 = M::pack4(pacc[mi][4 * i4], pacc[mi][4 * i4 + 1], pacc[mi][4 * i4 + 2],
-                                   pacc[mi][4 * i4 + 3]);
-          *(typename M::V4*)(ds_lds + row * C::DS_ROWB + swz<8>(row, 4 * mi + i4) * 16 + 8 * g) = h4;
-        }
-    }
-    __syncthreads();
-
-    // ---- dQ[:, d-block] = dS K, out through fp32 atomics ------------------------
-    {
-      const char* ds_lds = smem + C::OFF_DS;
-      float* dq_row0 = a.dq_acc + ((ws_row0 + i0) * a.heads_q + hq) * D + dq_db * 32 + l32;
-#pragma unroll
-      for (int n = 0; n < C::DQ_TILES; n++) {
-        const int mi = wave / C::DBLK + n * (4 / C::DBLK);
-        f32x16 acc;
-#pragma unroll
-        for (int i = 0; i < 16; i++) acc[i] = 0.f;
-#pragma unroll
-        for (int ks = 0; ks < C::BN / 16; ks++) {
-          const int row = ks * 16 + 8 * g + (i16 >> 2);
-          const int ch = 4 * mi + 2 * (u & 1) + ((i16 & 3) >> 1);
-          const int half = (i16 & 1) * 8;
-          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-              (lds_s16x4*)(ds_lds + row * C::DS_ROWB + swz<8>(row, ch) * 16 + half));
-          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-              (lds_s16x4*)(ds_lds + (row + 4) * C::DS_ROWB + swz<8>(row + 4, ch) * 16 + half));
-          const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-          V8 af;
-          __builtin_memcpy(&af, &both, 16);
-          acc = M::mfma32(af, ktf[ks], acc);
-        }
-#pragma unroll
         for (int i = 0; i < 16; i++) {
-          const int r = mi * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
-          if (i0 + r < len_q) unsafeAtomicAdd(dq_row0 + (int64_t)r * a.heads_q * D, acc[i]);
+          sacc[mi][i] = 0.f;
+          pacc[mi][i] = 0.f;
+        }
+#pragma unroll
+      for (int ks = 0; ks < C::KSTEPS; ks++) {
+#pragma unroll
+        for (int mi = 0; mi < C::MI; mi++) {
+          const int row = mi * 32 + l32;
+          const int off = row * C::ROWB + swz<C::CPR>(row, ks * 2 + g) * 16;
+          const V8 qa = *(const V8*)(q_lds + off);
+          const V8 da = *(const V8*)(do_lds + off);
+          sacc[mi] = M::mfma32(qa, kf[ks], sacc[mi]);
+          pacc[mi] = M::mfma32(da, vf[ks], pacc[mi]);
+        }
+      }
+
+      // ---- P and dS -----------------------------------------------------------
+      const bool full = i0 + C::BM - 1 < len_q && jw1 < len_k &&
+                        (a.wr < 0 || jw1 <= i0 + shift + a.wr) &&
+                        (a.wl < 0 || jw0 >= i0 + C::BM - 1 + shift - a.wl || jw1 < a.n_sink);
+#pragma unroll
+      for (int mi = 0; mi < C::MI; mi++) {
+#pragma unroll
+        for (int i4 = 0; i4 < 4; i4++) {
+          const int rbase = mi * 32 + 8 * i4 + 4 * g;
+          const f32x4 l4 = *(const f32x4*)(lse_lds + rbase);
+          const f32x4 d4 = *(const f32x4*)(delta_lds + rbase);
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            const int i = 4 * i4 + e;
+            float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[mi][i], a.scale_log2, -l4[e]));
+            if (!full) {
+              const int rel = jc - (i0 + rbase + e) - shift;  // offset from the aligned diagonal
+              const bool ok = jc < len_k && (a.wr < 0 || rel <= a.wr) &&
+                              (a.wl < 0 || rel >= -a.wl || jc < a.n_sink);
+              p = ok ? p : 0.f;  // rows past the end already have lse = +inf
+            }
+            sacc[mi][i] = p;
+            pacc[mi][i] = p * (pacc[mi][i] - d4[e]);
+          }
+        }
+      }
+
+      // ---- dV^T += dO^T P ; dK^T += Q^T dS --------------------------------------
+#pragma unroll
+      for (int ks = 0; ks < C::BM / 16; ks++) {
+        const int mi = ks >> 1;
+        float pv[8], dsv[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+          pv[j] = sacc[mi][8 * (ks & 1) + j];
+          dsv[j] = pacc[mi][8 * (ks & 1) + j];
+        }
+        const V8 pb = M::pack(pv);
+        const V8 dsb = M::pack(dsv);
+        const int row = ks * 16 + 4 * g + (i16 >> 2);
+#pragma unroll
+        for (int d = 0; d < C::DBLK; d++) {
+          const int ch = 4 * d + 2 * (u & 1) + ((i16 & 3) >> 1);
+          const int half = (i16 & 1) * 8;
+          const int off0 = row * C::ROWB + swz<C::CPR>(row, ch) * 16 + half;
+          const int off1 = (row + 8) * C::ROWB + swz<C::CPR>(row + 8, ch) * 16 + half;
+          dv_acc[d] = M::mfma32(tr_pair<V8>(do_lds + off0, do_lds + off1), pb, dv_acc[d]);
+          dk_acc[d] = M::mfma32(tr_pair<V8>(q_lds + off0, q_lds + off1), dsb, dk_acc[d]);
         }
       }
     }
@@ -387,8 +304,244 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(const AttnArgs a) {
   }
 }
 
-// delta[h][row] = sum_d dO * O ; zero the fp32 dQ accumulator.  One 16-lane (D=128) or
-// 8-lane (D=64) group per (row, head).
+// ============================================================================
+// dQ
+// ============================================================================
+template <int D>
+struct DqCfg {
+  static constexpr int BM = 128;  // query rows per block
+  static constexpr int BN = 64;   // keys per step
+  static constexpr int THREADS = 256;
+  static constexpr int KSTEPS = D / 16;
+  static constexpr int DBLK = D / 32;
+  static constexpr int CPR = D / 8;
+  static constexpr int ROWB = D * 2;
+  static constexpr int CH = BN * CPR / THREADS;
+  static constexpr int TILE = BN * ROWB;
+  static constexpr int OFF_K = 0;         // 2 buffers
+  static constexpr int OFF_V = 2 * TILE;  // 2 buffers
+  static constexpr int SMEM = 4 * TILE;
+  static constexpr int O_STRIDE = D * 2 + 16;
+  static_assert(SMEM >= 4 * 32 * O_STRIDE, "epilogue staging must fit");
+};
+
+template <typename T, int D>
+__global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const AttnArgs a) {
+  using C = DqCfg<D>;
+  using M = Mma<T>;
+  using V8 = typename M::V8;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+
+  const int wid = logical_block_id(a.n_work);
+  if (wid < 0) return;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int l32 = lane & 31;
+  const int g = lane >> 5;
+  const int i16 = lane & 15;
+  const int u = lane >> 4;
+
+  const int hg = wid % a.group;
+  int rest = wid / a.group;
+  const int slot = rest % a.n_tile;
+  rest /= a.n_tile;
+  const int hk = rest % a.heads_kv;
+  const int hq = hk * a.group + hg;
+  SeqInfo s;
+  int qt;
+  if (a.cu_q) {
+    if (!locate_packed(a, slot, C::BM, false, s, qt)) return;
+  } else {
+    s.batch_idx = rest / a.heads_kv;
+    s.q_row0 = s.k_row0 = 0;
+    s.len_q = a.seqlen_q;
+    s.len_k = a.seqlen_k;
+    qt = slot;
+  }
+  const int b = s.batch_idx;
+  const int len_q = s.len_q, len_k = s.len_k;
+  const int i0 = qt * C::BM;
+  if (i0 >= len_q) return;
+
+  const T* q_ptr = (const T*)a.q + b * a.q_st[0] + s.q_row0 * a.q_st[1] + hq * a.q_st[2];
+  const T* do_ptr = (const T*)a.dout + b * a.do_st[0] + s.q_row0 * a.do_st[1] + hq * a.do_st[2];
+  const T* k_ptr = (const T*)a.k + b * a.k_st[0] + s.k_row0 * a.k_st[1] + hk * a.k_st[2];
+  const T* v_ptr = (const T*)a.v + b * a.v_st[0] + s.k_row0 * a.v_st[1] + hk * a.v_st[2];
+  T* dq_ptr = (T*)a.dq + b * a.dq_st[0] + s.q_row0 * a.dq_st[1] + hq * a.dq_st[2];
+  const int64_t ws_row0 = a.cu_q ? s.q_row0 : (int64_t)b * a.seqlen_q;
+
+  // ---- key tiles this block visits (same rule as the forward kernel) -----------
+  const int i_last = min(i0 + C::BM, len_q) - 1;
+  const int lo_blk = row_bounds(a, i0, len_q, len_k).lo;
+  const int hi_blk = row_bounds(a, i_last, len_q, len_k).hi;
+  const bool band = hi_blk >= lo_blk;
+  const int t_lo = band ? lo_blk / C::BN : (1 << 29);
+  const int n_band = band ? hi_blk / C::BN - t_lo + 1 : 0;
+  const int sink_keys = max(0, min(min(a.n_sink, hi_blk + 1), lo_blk));
+  const int n_sink_t = min((sink_keys + C::BN - 1) / C::BN, t_lo);
+  const int n_tiles = n_sink_t + n_band;
+  auto tile_of = [&](int it) { return it < n_sink_t ? it : t_lo + (it - n_sink_t); };
+
+  const int r0 = i0 + wave * 32;
+  const int iq = r0 + l32;
+  const RowBounds rb = row_bounds(a, iq, len_q, len_k);
+  const bool wave_valid = r0 < len_q;
+  const bool wave_rows_full = r0 + 31 < len_q;
+  const RowBounds wb_first = row_bounds(a, r0, len_q, len_k);
+  const RowBounds wb_last = row_bounds(a, min(r0 + 31, len_q - 1), len_q, len_k);
+
+  // Q / dO fragments (B operands): lane = query column, 8 consecutive d per k-step
+  V8 qf[C::KSTEPS], dof[C::KSTEPS];
+  float lse2 = __builtin_inff(), delta = 0.f;
+  if (iq < len_q) {
+#pragma unroll
+    for (int ks = 0; ks < C::KSTEPS; ks++) {
+      qf[ks] = *(const V8*)(q_ptr + (int64_t)iq * a.q_st[1] + ks * 16 + g * 8);
+      dof[ks] = *(const V8*)(do_ptr + (int64_t)iq * a.do_st[1] + ks * 16 + g * 8);
+    }
+    const float l = a.lse[b * a.lse_st[0] + hq * a.lse_st[1] + (s.q_row0 + iq) * a.lse_st[2]];
+    lse2 = (l == -__builtin_inff()) ? __builtin_inff() : l * kLog2e;
+    delta = a.delta[(int64_t)hq * a.rows_q + ws_row0 + iq];
+  } else {
+#pragma unroll
+    for (int ks = 0; ks < C::KSTEPS; ks++) {
+      qf[ks] = V8{0, 0, 0, 0, 0, 0, 0, 0};
+      dof[ks] = V8{0, 0, 0, 0, 0, 0, 0, 0};
+    }
+  }
+
+  f32x16 dq_acc[C::DBLK];
+#pragma unroll
+  for (int d = 0; d < C::DBLK; d++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) dq_acc[d][i] = 0.f;
+
+  u32x4 kreg[C::CH], vreg[C::CH];
+  auto load_tile = [&](int tile) {
+    const int j0 = tile * C::BN;
+#pragma unroll
+    for (int n = 0; n < C::CH; n++) {
+      const int c = tid + n * C::THREADS;
+      const int row = c / C::CPR, col = (c % C::CPR) * 8;
+      if (j0 + row < len_k) {
+        kreg[n] = *(const u32x4*)(k_ptr + (int64_t)(j0 + row) * a.k_st[1] + col);
+        vreg[n] = *(const u32x4*)(v_ptr + (int64_t)(j0 + row) * a.v_st[1] + col);
+      } else {
+        kreg[n] = u32x4{0, 0, 0, 0};
+        vreg[n] = u32x4{0, 0, 0, 0};
+      }
+    }
+  };
+  auto store_tile = [&](int buf) {
+#pragma unroll
+    for (int n = 0; n < C::CH; n++) {
+      const int c = tid + n * C::THREADS;
+      const int row = c / C::CPR, ch = c % C::CPR;
+      const int off = row * C::ROWB + swz<C::CPR>(row, ch) * 16;
+      *(u32x4*)(smem + C::OFF_K + buf * C::TILE + off) = kreg[n];
+      *(u32x4*)(smem + C::OFF_V + buf * C::TILE + off) = vreg[n];
+    }
+  };
+
+  if (n_tiles > 0) {
+    load_tile(tile_of(0));
+    store_tile(0);
+  }
+  __syncthreads();
+
+  for (int it = 0; it < n_tiles; it++) {
+    const int buf = it & 1;
+    const int j0 = tile_of(it) * C::BN;
+    const int j1 = j0 + C::BN - 1;
+    if (it + 1 < n_tiles) load_tile(tile_of(it + 1));
+
+    const bool needed =
+        wave_valid && j0 <= wb_last.hi && (j1 >= wb_first.lo || j0 < a.n_sink);
+    if (needed) {
+      const char* k_lds = smem + C::OFF_K + buf * C::TILE;
+      const char* v_lds = smem + C::OFF_V + buf * C::TILE;
+      // S^T = K Q^T and dP^T = V dO^T (rows = keys, lane = query column)
+      f32x16 sacc[2], pacc[2];
+#pragma unroll
+      for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+          sacc[t][i] = 0.f;
+          pacc[t][i] = 0.f;
+        }
+#pragma unroll
+      for (int ks = 0; ks < C::KSTEPS; ks++) {
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+          const int row = t * 32 + l32;
+          const int off = row * C::ROWB + swz<C::CPR>(row, ks * 2 + g) * 16;
+          sacc[t] = M::mfma32(*(const V8*)(k_lds + off), qf[ks], sacc[t]);
+          pacc[t] = M::mfma32(*(const V8*)(v_lds + off), dof[ks], pacc[t]);
+        }
+      }
+      const bool full = wave_rows_full && j1 <= wb_first.hi &&
+                        (j0 >= wb_last.lo || j1 < a.n_sink);
+#pragma unroll
+      for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+          float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[t][i], a.scale_log2, -lse2));
+          if (!full) {
+            const int j = j0 + t * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
+            const bool ok = j <= rb.hi && (j >= rb.lo || j < a.n_sink);
+            p = ok ? p : 0.f;
+          }
+          pacc[t][i] = p * (pacc[t][i] - delta);
+        }
+      // dQ^T[d, query] += K^T dS^T
+      const int rlane = 4 * g + (i16 >> 2);
+      const int half = (i16 & 1) * 8;
+#pragma unroll
+      for (int s4 = 0; s4 < 4; s4++) {
+        float dsv[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) dsv[j] = pacc[s4 >> 1][8 * (s4 & 1) + j];
+        const V8 dsb = M::pack(dsv);
+        const int row = s4 * 16 + rlane;
+#pragma unroll
+        for (int d = 0; d < C::DBLK; d++) {
+          const int ch = 4 * d + 2 * (u & 1) + ((i16 & 3) >> 1);
+          const int off0 = row * C::ROWB + swz<C::CPR>(row, ch) * 16 + half;
+          const int off1 = (row + 8) * C::ROWB + swz<C::CPR>(row + 8, ch) * 16 + half;
+          dq_acc[d] = M::mfma32(tr_pair<V8>(k_lds + off0, k_lds + off1), dsb, dq_acc[d]);
+        }
+      }
+    }
+    if (it + 1 < n_tiles) store_tile(buf ^ 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue: dq = scale * acc, transposed through LDS for 16-byte stores ------
+  char* stage = smem + wave * 32 * C::O_STRIDE;
+#pragma unroll
+  for (int d = 0; d < C::DBLK; d++)
+#pragma unroll
+    for (int i4 = 0; i4 < 4; i4++) {
+      const auto h4 = M::pack4(dq_acc[d][4 * i4] * a.scale, dq_acc[d][4 * i4 + 1] * a.scale,
+                               dq_acc[d][4 * i4 + 2] * a.scale, dq_acc[d][4 * i4 + 3] * a.scale);
+      *(typename M::V4*)(stage + l32 * C::O_STRIDE + (d * 32 + 8 * i4 + 4 * g) * 2) = h4;
+    }
+  __syncthreads();
+#pragma unroll
+  for (int n = 0; n < 32 * C::CPR / 64; n++) {
+    const int c = lane + n * 64;
+    const int row = c / C::CPR, col = (c % C::CPR) * 8;
+    if (r0 + row < len_q) {
+      const u32x4 val = *(const u32x4*)(stage + row * C::O_STRIDE + col * 2);
+      *(u32x4*)(dq_ptr + (int64_t)(r0 + row) * a.dq_st[1] + col) = val;
+    }
+  }
+}
+
+// ============================================================================
+// delta[h][row] = sum_d dO * O.  One 16-lane (D=128) or 8-lane (D=64) group per (row, head).
+// ============================================================================
 template <typename T, int D>
 __global__ __launch_bounds__(256) void attn_bwd_prep_kernel(const AttnArgs a) {
   constexpr int LPR = D / 8;
@@ -415,66 +568,65 @@ __global__ __launch_bounds__(256) void attn_bwd_prep_kernel(const AttnArgs a) {
 #pragma unroll
   for (int m = LPR / 2; m >= 1; m >>= 1) acc += __shfl_xor(acc, m, 64);
   if (c == 0) a.delta[(int64_t)h * a.rows_q + row] = acc;
-  f32x4* z = (f32x4*)(a.dq_acc + unit * D + c);
-  z[0] = f32x4{0.f, 0.f, 0.f, 0.f};
-  z[1] = f32x4{0.f, 0.f, 0.f, 0.f};
 }
 
-template <typename T, int D>
-__global__ __launch_bounds__(256) void attn_bwd_post_kernel(const AttnArgs a) {
-  constexpr int LPR = D / 8;
-  const int64_t unit = ((int64_t)blockIdx.x * 256 + threadIdx.x) / LPR;
-  const int c = (threadIdx.x % LPR) * 8;
-  if (unit >= a.rows_q * a.heads_q) return;
-  const int h = (int)(unit % a.heads_q);
-  const int64_t row = unit / a.heads_q;
-  int64_t off;
-  if (a.cu_q) {
-    off = row * a.dq_st[1];
-  } else {
-    off = (row / a.seqlen_q) * a.dq_st[0] + (row % a.seqlen_q) * a.dq_st[1];
+template <typename Kern>
+int set_smem(Kern kern, int bytes, bool& configured, const char* what) {
+  if (!configured) {  // benign race: the attribute call is idempotent
+    hipError_t e =
+        hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e != hipSuccess) return fail(RSWA_ERR_LAUNCH, "%s: set smem: %s", what, hipGetErrorString(e));
+    configured = true;
   }
-  const f32x4* src = (const f32x4*)(a.dq_acc + unit * D + c);
-  const f32x4 x = src[0], y = src[1];
-  float f[8] = {x[0] * a.scale, x[1] * a.scale, x[2] * a.scale, x[3] * a.scale,
-                y[0] * a.scale, y[1] * a.scale, y[2] * a.scale, y[3] * a.scale};
-  *(typename Mma<T>::V8*)((T*)a.dq + off + h * a.dq_st[2] + c) = Mma<T>::pack(f);
+  return RSWA_OK;
 }
 
 template <typename T, int D>
 int launch_bwd(AttnArgs& a, hipStream_t stream, int phases) {
-  using C = BwdCfg<D>;
   const int64_t units = a.rows_q * a.heads_q;
-  const unsigned ew_blocks = (unsigned)ceil_div(units * (D / 8), 256);
   if (units > 0 && (phases & RSWA_BWD_PREP)) {
-    hipLaunchKernelGGL((attn_bwd_prep_kernel<T, D>), dim3(ew_blocks), dim3(256), 0, stream, a);
+    const unsigned blocks = (unsigned)ceil_div(units * (D / 8), 256);
+    hipLaunchKernelGGL((attn_bwd_prep_kernel<T, D>), dim3(blocks), dim3(256), 0, stream, a);
     int rc = check_launch("attn_bwd prep");
     if (rc != RSWA_OK) return rc;
   }
-  if (a.cu_q) {
-    a.n_tile = (int)(ceil_div(a.rows_k, C::BN) + a.batch);
-    a.n_work = a.n_tile * a.heads_kv;
-  } else {
-    a.n_tile = (int)ceil_div(a.seqlen_k, C::BN);
-    a.n_work = a.n_tile * a.heads_kv * a.batch;
-  }
-  if (a.n_work > 0 && (phases & RSWA_BWD_MAIN)) {
-    auto kern = attn_bwd_kernel<T, D>;
-    static bool configured = false;  // benign race: the attribute call is idempotent
-    if (!configured) {
-      hipError_t e = hipFuncSetAttribute((const void*)kern,
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
-      if (e != hipSuccess)
-        return fail(RSWA_ERR_LAUNCH, "attn_bwd: set smem: %s", hipGetErrorString(e));
-      configured = true;
+  if (phases & RSWA_BWD_DKDV) {
+    using C = DkvCfg<D>;
+    if (a.cu_q) {
+      a.n_tile = (int)(ceil_div(a.rows_k, C::BN) + a.batch);
+      a.n_work = a.n_tile * a.heads_kv;
+    } else {
+      a.n_tile = (int)ceil_div(a.seqlen_k, C::BN);
+      a.n_work = a.n_tile * a.heads_kv * a.batch;
     }
-    hipLaunchKernelGGL(kern, dim3(padded_grid(a.n_work)), dim3(C::THREADS), C::SMEM, stream, a);
-    int rc = check_launch("attn_bwd main");
-    if (rc != RSWA_OK) return rc;
+    if (a.n_work > 0) {
+      auto kern = attn_bwd_dkdv_kernel<T, D>;
+      static bool configured = false;
+      int rc = set_smem(kern, C::SMEM, configured, "attn_bwd dkdv");
+      if (rc != RSWA_OK) return rc;
+      hipLaunchKernelGGL(kern, dim3(padded_grid(a.n_work)), dim3(C::THREADS), C::SMEM, stream, a);
+      rc = check_launch("attn_bwd dkdv");
+      if (rc != RSWA_OK) return rc;
+    }
   }
-  if (units > 0 && (phases & RSWA_BWD_POST)) {
-    hipLaunchKernelGGL((attn_bwd_post_kernel<T, D>), dim3(ew_blocks), dim3(256), 0, stream, a);
-    return check_launch("attn_bwd post");
+  if (phases & RSWA_BWD_DQ) {
+    using C = DqCfg<D>;
+    if (a.cu_q) {
+      a.n_tile = (int)(ceil_div(a.rows_q, C::BM) + a.batch);
+      a.n_work = a.n_tile * a.heads_q;
+    } else {
+      a.n_tile = (int)ceil_div(a.seqlen_q, C::BM);
+      a.n_work = a.n_tile * a.heads_q * a.batch;
+    }
+    if (a.n_work > 0) {
+      auto kern = attn_bwd_dq_kernel<T, D>;
+      static bool configured = false;
+      int rc = set_smem(kern, C::SMEM, configured, "attn_bwd dq");
+      if (rc != RSWA_OK) return rc;
+      hipLaunchKernelGGL(kern, dim3(padded_grid(a.n_work)), dim3(C::THREADS), C::SMEM, stream, a);
+      rc = check_launch("attn_bwd dq");
+      if (rc != RSWA_OK) return rc;
+    }
   }
   return RSWA_OK;
 }
@@ -497,5 +649,5 @@ extern "C" int rswa_attn_bwd_phases(const rswa_attn_params* p, void* stream, int
 }
 
 extern "C" int rswa_attn_bwd(const rswa_attn_params* p, void* stream) {
-  return rswa_attn_bwd_phases(p, stream, RSWA_BWD_PREP | RSWA_BWD_MAIN | RSWA_BWD_POST);
+  return rswa_attn_bwd_phases(p, stream, RSWA_BWD_PREP | RSWA_BWD_DKDV | RSWA_BWD_DQ);
 }

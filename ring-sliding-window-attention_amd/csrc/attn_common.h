@@ -29,7 +29,6 @@ struct AttnArgs {
   void* dq;
   void* dk;
   void* dv;
-  float* dq_acc;  // fp32 [rows_q, heads_q, head_dim] packed, inside the workspace
   float* delta;   // fp32 [heads_q, rows_q] packed, inside the workspace
   const int32_t* cu_q;
   const int32_t* cu_k;
@@ -141,6 +140,20 @@ struct Mma<_Float16> {
 };
 
 typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+
+// XOR swizzle of 16-byte chunks inside an LDS tile whose rows hold CH chunks (8 or 16).
+// It makes both access patterns used by the kernels bank-conflict free: 16 consecutive
+// rows at one logical chunk (MFMA row fragments, 16-byte reads) and 4 consecutive rows x
+// 4 consecutive chunks (one phase of the transposing 8-byte reads).
+template <int CH>
+__device__ __forceinline__ int swz(int row, int chunk) {
+  if constexpr (CH == 16) {
+    return chunk ^ (((row & 3) << 2) | ((row >> 2) & 3));
+  } else {
+    static_assert(CH == 8, "rows of 8 or 16 chunks");
+    return chunk ^ ((((row >> 1) & 1) << 2) | ((row >> 2) & 3));
+  }
+}
 
 // max / sum across the two half-waves (lane l <-> lane l ^ 32).
 __device__ __forceinline__ float halfwave_max(float x) {

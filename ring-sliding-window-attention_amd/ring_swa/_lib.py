@@ -13,7 +13,8 @@ from ctypes import (POINTER, Structure, c_char_p, c_float, c_int, c_int32, c_int
 import torch
 
 _PKG_ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-LIB_PATH = os.path.join(_PKG_ROOT, "lib", "librswa.so")
+# RSWA_LIBRARY lets a deployment point at a library built elsewhere.
+LIB_PATH = os.environ.get("RSWA_LIBRARY") or os.path.join(_PKG_ROOT, "lib", "librswa.so")
 
 RSWA_BF16, RSWA_F16, RSWA_F32, RSWA_F64 = 0, 1, 2, 3
 _DTYPES = {

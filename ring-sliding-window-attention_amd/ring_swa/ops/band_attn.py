@@ -148,7 +148,7 @@ def attn_bwd(
 
     ``workspace`` (uint8, at least ``rswa_attn_bwd_workspace_bytes``) may be supplied to
     avoid the per-call scratch allocation; ``phases`` is the bit mask of
-    ``rswa_attn_bwd_phases`` (1 prep, 2 main, 4 post) for profiling."""
+    ``rswa_attn_bwd_phases`` (1 prep, 2 dk/dv kernel, 4 dq kernel) for profiling."""
     packed = cu_seqlens_q is not None
     _check_qkv(q, k, v, packed)
     dev = _lib.require_device(q, k, v, o, softmax_lse, do, dq, dk, dv)
