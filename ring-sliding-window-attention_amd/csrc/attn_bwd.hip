@@ -52,7 +52,6 @@ struct DkvCfg {
   static constexpr int DBLK = D / 32;
   static constexpr int CPR = D / 8;   // 16-byte chunks per row
   static constexpr int ROWB = D * 2;  // bytes per row
-  static constexpr int QCH = BM * CPR / THREADS;
   static constexpr int Q_TILE = BM * ROWB;
   static constexpr int OFF_Q = 0;            // 2 buffers
   static constexpr int OFF_DO = 2 * Q_TILE;  // 2 buffers
@@ -137,30 +136,33 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
       dv_acc[d][i] = 0.f;
     }
 
-  // ---- tile movement: Q, dO, lse, delta of iteration `it` ---------------------
-  u32x4 qreg[C::QCH], doreg[C::QCH];
+  // ---- lane-constant LDS offsets (swizzle folded: varying parts are XOR / immediates) ----
+  // row fragments of Q / dO (16-byte reads): row = 32 mi + l32, chunk = 2 ks + g
+  //   offset = (a_row ^ (ks << 5)) + mi * 32 * ROWB
+  const int a_row = l32 * C::ROWB + ((g ^ swz_f<C::CPR>(l32)) << 4);
+  // transposing reads of Q / dO: rows 16 ks + 4 g + (i16 >> 2) and + 8, chunk = 4 d + lp
+  //   offset = (t_row{0,1} ^ (d << 6)) + ks * 16 * ROWB
+  const int rl = 4 * g + (i16 >> 2);
+  const int lp = 2 * (u & 1) + ((i16 & 3) >> 1);
+  const int t_row0 = rl * C::ROWB + ((lp ^ swz_f<C::CPR>(rl)) << 4) + (i16 & 1) * 8;
+  const int t_row1 = (rl + 8) * C::ROWB + ((lp ^ swz_f<C::CPR>(rl + 8)) << 4) + (i16 & 1) * 8;
+
+  // ---- tile movement: Q, dO straight into LDS; lse, delta through one register ----
   float streg = 0.f;
   auto iter_coords = [&](int it, int& hq, int& i0) {
     hq = hk * a.group + it / n_qt;
     i0 = (qt_lo + it % n_qt) * C::BM;
   };
-  auto load_iter = [&](int it) {
+  auto load_iter = [&](int it, int buf) {
     int hq, i0;
     iter_coords(it, hq, i0);
-    const T* q_ptr = (const T*)a.q + b * a.q_st[0] + s.q_row0 * a.q_st[1] + hq * a.q_st[2];
-    const T* do_ptr = (const T*)a.dout + b * a.do_st[0] + s.q_row0 * a.do_st[1] + hq * a.do_st[2];
-#pragma unroll
-    for (int n = 0; n < C::QCH; n++) {
-      const int c = tid + n * C::THREADS;
-      const int row = c / C::CPR, ch = c % C::CPR;
-      if (i0 + row < len_q) {
-        qreg[n] = *(const u32x4*)(q_ptr + (int64_t)(i0 + row) * a.q_st[1] + ch * 8);
-        doreg[n] = *(const u32x4*)(do_ptr + (int64_t)(i0 + row) * a.do_st[1] + ch * 8);
-      } else {
-        qreg[n] = u32x4{0, 0, 0, 0};
-        doreg[n] = u32x4{0, 0, 0, 0};
-      }
-    }
+    const T* q_ptr = (const T*)a.q + b * a.q_st[0] + (s.q_row0 + i0) * a.q_st[1] + hq * a.q_st[2];
+    const T* do_ptr =
+        (const T*)a.dout + b * a.do_st[0] + (s.q_row0 + i0) * a.do_st[1] + hq * a.do_st[2];
+    g2lds_tile<T, D, C::BM, C::THREADS>(q_ptr, a.q_st[1], len_q - i0,
+                                         smem + C::OFF_Q + buf * C::Q_TILE, tid);
+    g2lds_tile<T, D, C::BM, C::THREADS>(do_ptr, a.do_st[1], len_q - i0,
+                                         smem + C::OFF_DO + buf * C::Q_TILE, tid);
     if (tid < C::BM) {
       // lse in base-2 units; rows that must contribute nothing get +inf (P = 0)
       const int i = i0 + tid;
@@ -175,21 +177,13 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
       streg = (i < len_q) ? a.delta[(int64_t)hq * a.rows_q + ws_row0 + i] : 0.f;
     }
   };
-  auto store_iter = [&](int buf) {
-#pragma unroll
-    for (int n = 0; n < C::QCH; n++) {
-      const int c = tid + n * C::THREADS;
-      const int row = c / C::CPR, ch = c % C::CPR;
-      const int off = row * C::ROWB + swz<C::CPR>(row, ch) * 16;
-      *(u32x4*)(smem + C::OFF_Q + buf * C::Q_TILE + off) = qreg[n];
-      *(u32x4*)(smem + C::OFF_DO + buf * C::Q_TILE + off) = doreg[n];
-    }
+  auto store_stats = [&](int buf) {
     if (tid < 2 * C::BM) *(float*)(smem + C::OFF_ST + buf * 2 * C::BM * 4 + tid * 4) = streg;
   };
 
   if (n_iter > 0) {
-    load_iter(0);
-    store_iter(0);
+    load_iter(0, 0);
+    store_stats(0);
   }
   __syncthreads();
 
@@ -197,7 +191,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
     const int buf = it & 1;
     int hq, i0;
     iter_coords(it, hq, i0);
-    if (it + 1 < n_iter) load_iter(it + 1);
+    if (it + 1 < n_iter) load_iter(it + 1, buf ^ 1);
     const char* q_lds = smem + C::OFF_Q + buf * C::Q_TILE;
     const char* do_lds = smem + C::OFF_DO + buf * C::Q_TILE;
     const float* lse_lds = (const float*)(smem + C::OFF_ST + buf * 2 * C::BM * 4);
@@ -220,12 +214,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
         }
 #pragma unroll
       for (int ks = 0; ks < C::KSTEPS; ks++) {
+        const int off = a_row ^ (ks << 5);
 #pragma unroll
         for (int mi = 0; mi < C::MI; mi++) {
-          const int row = mi * 32 + l32;
-          const int off = row * C::ROWB + swz<C::CPR>(row, ks * 2 + g) * 16;
-          const V8 qa = *(const V8*)(q_lds + off);
-          const V8 da = *(const V8*)(do_lds + off);
+          const V8 qa = *(const V8*)(q_lds + off + mi * 32 * C::ROWB);
+          const V8 da = *(const V8*)(do_lds + off + mi * 32 * C::ROWB);
           sacc[mi] = M::mfma32(qa, kf[ks], sacc[mi]);
           pacc[mi] = M::mfma32(da, vf[ks], pacc[mi]);
         }
@@ -235,6 +228,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
       const bool full = i0 + C::BM - 1 < len_q && jw1 < len_k &&
                         (a.wr < 0 || jw1 <= i0 + shift + a.wr) &&
                         (a.wl < 0 || jw0 >= i0 + C::BM - 1 + shift - a.wl || jw1 < a.n_sink);
+      // key position relative to the aligned diagonal of query row i0: rel(i) = rel0 - (i - i0)
+      const int rel0 = jc - i0 - shift;
+      const int rel_hi = (a.wr < 0) ? (1 << 30) : a.wr;
+      const int rel_lo = (a.wl < 0 || jc < a.n_sink) ? -(1 << 30) : -a.wl;
+      const bool col_ok = jc < len_k;
 #pragma unroll
       for (int mi = 0; mi < C::MI; mi++) {
 #pragma unroll
@@ -247,9 +245,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
             const int i = 4 * i4 + e;
             float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[mi][i], a.scale_log2, -l4[e]));
             if (!full) {
-              const int rel = jc - (i0 + rbase + e) - shift;  // offset from the aligned diagonal
-              const bool ok = jc < len_k && (a.wr < 0 || rel <= a.wr) &&
-                              (a.wl < 0 || rel >= -a.wl || jc < a.n_sink);
+              const int rel = rel0 - (rbase + e);
+              const bool ok = col_ok & (rel <= rel_hi) & (rel >= rel_lo);
               p = ok ? p : 0.f;  // rows past the end already have lse = +inf
             }
             sacc[mi][i] = p;
@@ -270,20 +267,17 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
         }
         const V8 pb = M::pack(pv);
         const V8 dsb = M::pack(dsv);
-        const int row = ks * 16 + 4 * g + (i16 >> 2);
 #pragma unroll
         for (int d = 0; d < C::DBLK; d++) {
-          const int ch = 4 * d + 2 * (u & 1) + ((i16 & 3) >> 1);
-          const int half = (i16 & 1) * 8;
-          const int off0 = row * C::ROWB + swz<C::CPR>(row, ch) * 16 + half;
-          const int off1 = (row + 8) * C::ROWB + swz<C::CPR>(row + 8, ch) * 16 + half;
+          const int off0 = (t_row0 ^ (d << 6)) + ks * 16 * C::ROWB;
+          const int off1 = (t_row1 ^ (d << 6)) + ks * 16 * C::ROWB;
           dv_acc[d] = M::mfma32(tr_pair<V8>(do_lds + off0, do_lds + off1), pb, dv_acc[d]);
           dk_acc[d] = M::mfma32(tr_pair<V8>(q_lds + off0, q_lds + off1), dsb, dk_acc[d]);
         }
       }
     }
 
-    if (it + 1 < n_iter) store_iter(buf ^ 1);
+    if (it + 1 < n_iter) store_stats(buf ^ 1);
     __syncthreads();
   }
 
@@ -326,7 +320,7 @@ struct DqCfg {
 };
 
 template <typename T, int D>
-__global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const AttnArgs a) {
+__global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
   using C = DqCfg<D>;
   using M = Mma<T>;
   using V8 = typename M::V8;

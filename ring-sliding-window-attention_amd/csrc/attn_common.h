@@ -141,17 +141,51 @@ struct Mma<_Float16> {
 
 typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
 
-// XOR swizzle of 16-byte chunks inside an LDS tile whose rows hold CH chunks (8 or 16).
-// It makes both access patterns used by the kernels bank-conflict free: 16 consecutive
-// rows at one logical chunk (MFMA row fragments, 16-byte reads) and 4 consecutive rows x
-// 4 consecutive chunks (one phase of the transposing 8-byte reads).
+// XOR swizzle of 16-byte chunks inside an LDS tile whose rows hold CH chunks (8 or 16):
+// chunk c of row r is stored at chunk position c ^ swz_f<CH>(r).  It makes both access
+// patterns used by the kernels bank-conflict free: 16 consecutive rows at one logical
+// chunk (MFMA row fragments, 16-byte reads) and 4 consecutive rows x 4 consecutive chunks
+// (one phase of the transposing 8-byte reads).  swz_f only looks at the low 4 bits of the
+// row, so offsets of 16 rows (and of 32-row blocks) fold into immediate offsets.
 template <int CH>
-__device__ __forceinline__ int swz(int row, int chunk) {
+__device__ __forceinline__ int swz_f(int row) {
   if constexpr (CH == 16) {
-    return chunk ^ (((row & 3) << 2) | ((row >> 2) & 3));
+    return ((row & 3) << 2) | ((row >> 2) & 3);
   } else {
     static_assert(CH == 8, "rows of 8 or 16 chunks");
-    return chunk ^ ((((row >> 1) & 1) << 2) | ((row >> 2) & 3));
+    return (((row >> 1) & 1) << 2) | ((row >> 2) & 3);
+  }
+}
+template <int CH>
+__device__ __forceinline__ int swz(int row, int chunk) {
+  return chunk ^ swz_f<CH>(row);
+}
+
+typedef __attribute__((address_space(3))) void lds_void_t;
+typedef __attribute__((address_space(1))) const void glob_void_t;
+
+// Cooperative copy of a [ROWS x D] tile (row-major in global memory, `stride` elements
+// between rows) into a swizzled LDS tile with direct global->LDS loads
+// (global_load_lds_dwordx4: lane L of a wave lands at wave_base + 16 L): no staging
+// registers, no LDS store instructions.  Rows >= valid_rows repeat row valid_rows - 1
+// (finite data the mask never lets through); valid_rows must be >= 1.
+template <typename T, int D, int ROWS, int THREADS>
+__device__ __forceinline__ void g2lds_tile(const T* src, int64_t stride, int valid_rows,
+                                           char* lds_tile, int tid) {
+  constexpr int CPR = D / 8;
+  constexpr int RPI = 64 / CPR;  // rows per wave instruction
+  constexpr int NW = THREADS / 64;
+  constexpr int N = ROWS * CPR / THREADS;
+  static_assert(N * THREADS == ROWS * CPR, "tile must divide evenly");
+  const int lane = tid & 63, wave = tid >> 6;
+#pragma unroll
+  for (int n = 0; n < N; n++) {
+    const int slot = n * NW + wave;
+    const int row = slot * RPI + lane / CPR;
+    const int lc = (lane % CPR) ^ swz_f<CPR>(row);
+    const int rr = min(row, valid_rows - 1);
+    __builtin_amdgcn_global_load_lds((glob_void_t*)(src + (int64_t)rr * stride + lc * 8),
+                                     (lds_void_t*)(lds_tile + slot * 1024), 16, 0, 0);
   }
 }
 

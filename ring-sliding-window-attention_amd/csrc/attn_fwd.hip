@@ -36,7 +36,9 @@ struct FwdCfg {
 };
 
 template <typename T, int D>
-__global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs a) {
+// two blocks per CU (2 waves per SIMD): keeps everything in the 256 architectural VGPRs,
+// so no accumulator-register copies, and lets one wave's softmax overlap another's MFMAs
+__global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
   using C = FwdCfg<D>;
   using M = Mma<T>;
   using V8 = typename M::V8;
