@@ -3,9 +3,11 @@
 // Replaces flash-attn's backward as wrapped at ring_swa/ops/wrap_flash.py:276-429.
 // Three launches on the caller's stream:
 //   PREP : delta[h][row] = sum_d dO * O   (fp32, in the caller's workspace)
-//   DKDV : one block owns 128 keys of one (sequence, kv head) and walks the query tiles
-//          (64 rows) that can see them, for every q head of the GQA group; dK^T / dV^T
-//          stay in registers for the whole walk and are written once
+//   DKDV : one block (8 waves) owns 128 keys of one (sequence, kv head), keeps their K and
+//          V tiles in LDS and walks the query tiles (64 rows) that can see them, for every
+//          q head of the GQA group; wave (wk, wq) handles key columns 32 wk.. of query rows
+//          32 wq.. of each tile; dK^T / dV^T partials stay in registers for the whole walk,
+//          the two query halves are added through LDS at the end and written once
 //   DQ   : one block owns 128 queries of one (sequence, q head) and walks the key tiles
 //          (64 keys) it can see, like the forward kernel; dQ^T stays in registers
 // S and dP are computed in both main kernels (7 GEMM units instead of 5).  That costs
@@ -13,8 +15,8 @@
 // channel, which caps an atomic dQ far below the MFMA rate.  It also makes the result
 // run-to-run deterministic.
 //
-// DKDV per (query tile, wave); wave w owns key columns 32w..32w+31 (C layout: lane = key):
-//   S = Q K^T, dP = dO V^T      A = Q / dO row fragments from LDS, B = K / V fragments (regs)
+// DKDV per (query half-tile, wave) (C layout: lane = key):
+//   S = Q K^T, dP = dO V^T      A = Q / dO row fragments, B = K / V row fragments (all LDS)
 //   P = exp2(S*c - lse*log2e), dS = P * (dP - delta)
 //   dV^T += dO^T P, dK^T += Q^T dS   A = transposing LDS reads of dO / Q, B = P / dS (regs)
 // DQ per (key tile, wave); wave w owns query columns 32w..32w+31 (C layout: lane = query):
@@ -46,21 +48,27 @@ template <int D>
 struct DkvCfg {
   static constexpr int BM = 64;   // query rows per step
   static constexpr int BN = 128;  // keys per block
-  static constexpr int THREADS = 256;
-  static constexpr int MI = BM / 32;
+  static constexpr int THREADS = 512;  // 8 waves: 4 key groups x 2 query halves
   static constexpr int KSTEPS = D / 16;
   static constexpr int DBLK = D / 32;
   static constexpr int CPR = D / 8;   // 16-byte chunks per row
   static constexpr int ROWB = D * 2;  // bytes per row
   static constexpr int Q_TILE = BM * ROWB;
-  static constexpr int OFF_Q = 0;            // 2 buffers
-  static constexpr int OFF_DO = 2 * Q_TILE;  // 2 buffers
-  static constexpr int OFF_ST = 4 * Q_TILE;  // lse2[2][BM], delta[2][BM] fp32
+  static constexpr int KV_TILE = BN * ROWB;
+  static constexpr int OFF_K = 0;
+  static constexpr int OFF_V = KV_TILE;
+  static constexpr int OFF_Q = 2 * KV_TILE;            // 2 buffers
+  static constexpr int OFF_DO = OFF_Q + 2 * Q_TILE;    // 2 buffers
+  static constexpr int OFF_ST = OFF_DO + 2 * Q_TILE;   // lse2[2][BM], delta[2][BM] fp32
   static constexpr int SMEM = OFF_ST + 4 * BM * 4;
+  // end-of-walk reduction of the two query halves: per key group 2 matrices of
+  // DBLK x 16 registers x 64 lanes fp32
+  static constexpr int RED_PER_WK = 2 * DBLK * 16 * 64 * 4;
+  static_assert(4 * RED_PER_WK <= SMEM, "reduction staging must fit");
 };
 
 template <typename T, int D>
-__global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
+__global__ __launch_bounds__(512) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   using C = DkvCfg<D>;
   using M = Mma<T>;
   using V8 = typename M::V8;
@@ -71,6 +79,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
+  const int wk = wave & 3;   // key group: columns 32 wk .. 32 wk + 31 of the block's 128 keys
+  const int wq = wave >> 2;  // query half: rows 32 wq .. 32 wq + 31 of each 64-row tile
   const int l32 = lane & 31;
   const int g = lane >> 5;
   const int i16 = lane & 15;
@@ -98,8 +108,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   const int j_last = min(j0 + C::BN, len_k) - 1;
   const int shift = a.shift_explicit ? a.shift_val : len_k - len_q;
 
-  const T* k_ptr = (const T*)a.k + b * a.k_st[0] + s.k_row0 * a.k_st[1] + hk * a.k_st[2];
-  const T* v_ptr = (const T*)a.v + b * a.v_st[0] + s.k_row0 * a.v_st[1] + hk * a.v_st[2];
+  const T* k_ptr = (const T*)a.k + b * a.k_st[0] + (s.k_row0 + j0) * a.k_st[1] + hk * a.k_st[2];
+  const T* v_ptr = (const T*)a.v + b * a.v_st[0] + (s.k_row0 + j0) * a.v_st[1] + hk * a.v_st[2];
   T* dk_ptr = (T*)a.dk + b * a.dk_st[0] + s.k_row0 * a.dk_st[1] + hk * a.dk_st[2];
   T* dv_ptr = (T*)a.dv + b * a.dv_st[0] + s.k_row0 * a.dv_st[1] + hk * a.dv_st[2];
   const int64_t ws_row0 = a.cu_q ? s.q_row0 : (int64_t)b * a.seqlen_q;
@@ -112,20 +122,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   const int n_qt = (i_max >= i_min) ? i_max / C::BM - qt_lo + 1 : 0;
   const int n_iter = n_qt * a.group;
 
-  // ---- K / V fragments (B operands), resident for the whole walk --------------
-  const int jw0 = j0 + wave * 32;  // first key column of this wave
-  const int jc = jw0 + l32;        // this lane's key column
-  V8 kf[C::KSTEPS], vf[C::KSTEPS];
-#pragma unroll
-  for (int ks = 0; ks < C::KSTEPS; ks++) {
-    if (jc < len_k) {
-      kf[ks] = *(const V8*)(k_ptr + (int64_t)jc * a.k_st[1] + ks * 16 + g * 8);
-      vf[ks] = *(const V8*)(v_ptr + (int64_t)jc * a.v_st[1] + ks * 16 + g * 8);
-    } else {
-      kf[ks] = V8{0, 0, 0, 0, 0, 0, 0, 0};
-      vf[ks] = V8{0, 0, 0, 0, 0, 0, 0, 0};
-    }
-  }
+  const int jw0 = j0 + wk * 32;  // first key column of this wave
+  const int jc = jw0 + l32;      // this lane's key column
 
   f32x16 dk_acc[C::DBLK], dv_acc[C::DBLK];
 #pragma unroll
@@ -137,8 +135,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
     }
 
   // ---- lane-constant LDS offsets (swizzle folded: varying parts are XOR / immediates) ----
-  // row fragments of Q / dO (16-byte reads): row = 32 mi + l32, chunk = 2 ks + g
-  //   offset = (a_row ^ (ks << 5)) + mi * 32 * ROWB
+  // 16-byte row fragments: row = 32 blk + l32, chunk = 2 ks + g
+  //   offset = (a_row ^ (ks << 5)) + blk * 32 * ROWB      (Q / dO: blk = wq; K / V: blk = wk)
   const int a_row = l32 * C::ROWB + ((g ^ swz_f<C::CPR>(l32)) << 4);
   // transposing reads of Q / dO: rows 16 ks + 4 g + (i16 >> 2) and + 8, chunk = 4 d + lp
   //   offset = (t_row{0,1} ^ (d << 6)) + ks * 16 * ROWB
@@ -147,7 +145,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   const int t_row0 = rl * C::ROWB + ((lp ^ swz_f<C::CPR>(rl)) << 4) + (i16 & 1) * 8;
   const int t_row1 = (rl + 8) * C::ROWB + ((lp ^ swz_f<C::CPR>(rl + 8)) << 4) + (i16 & 1) * 8;
 
-  // ---- tile movement: Q, dO straight into LDS; lse, delta through one register ----
+  // ---- tile movement: everything lands in LDS directly; lse, delta via one register ----
   float streg = 0.f;
   auto iter_coords = [&](int it, int& hq, int& i0) {
     hq = hk * a.group + it / n_qt;
@@ -182,10 +180,15 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   };
 
   if (n_iter > 0) {
+    g2lds_tile<T, D, C::BN, C::THREADS>(k_ptr, a.k_st[1], len_k - j0, smem + C::OFF_K, tid);
+    g2lds_tile<T, D, C::BN, C::THREADS>(v_ptr, a.v_st[1], len_k - j0, smem + C::OFF_V, tid);
     load_iter(0, 0);
     store_stats(0);
   }
   __syncthreads();
+
+  const char* k_lds = smem + C::OFF_K + wk * 32 * C::ROWB;
+  const char* v_lds = smem + C::OFF_V + wk * 32 * C::ROWB;
 
   for (int it = 0; it < n_iter; it++) {
     const int buf = it & 1;
@@ -194,83 +197,79 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
     if (it + 1 < n_iter) load_iter(it + 1, buf ^ 1);
     const char* q_lds = smem + C::OFF_Q + buf * C::Q_TILE;
     const char* do_lds = smem + C::OFF_DO + buf * C::Q_TILE;
-    const float* lse_lds = (const float*)(smem + C::OFF_ST + buf * 2 * C::BM * 4);
+    const float* lse_lds = (const float*)(smem + C::OFF_ST + buf * 2 * C::BM * 4) + wq * 32;
     const float* delta_lds = lse_lds + C::BM;
 
-    // Does any (query of the tile, key of this wave) pair survive the mask?
-    const int i_end = min(i0 + C::BM, len_q) - 1;
+    // Does any (query of this wave's half-tile, key of this wave) pair survive the mask?
+    const int iw0 = i0 + wq * 32;
+    const int iw1 = min(iw0 + 32, len_q) - 1;
     const int jw1 = jw0 + 31;
-    const bool needed = jw0 < len_k && (a.wr < 0 || jw0 <= i_end + shift + a.wr) &&
-                        (a.wl < 0 || jw1 >= i0 + shift - a.wl || jw0 < a.n_sink);
+    const bool needed = iw0 < len_q && jw0 < len_k &&
+                        (a.wr < 0 || jw0 <= iw1 + shift + a.wr) &&
+                        (a.wl < 0 || jw1 >= iw0 + shift - a.wl || jw0 < a.n_sink);
     if (needed) {
       // ---- S = Q K^T and dP = dO V^T (rows = queries, lane = key column) ------
-      f32x16 sacc[C::MI], pacc[C::MI];
+      f32x16 sacc, pacc;
 #pragma unroll
-      for (int mi = 0; mi < C::MI; mi++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-          sacc[mi][i] = 0.f;
-          pacc[mi][i] = 0.f;
-        }
+      for (int i = 0; i < 16; i++) {
+        sacc[i] = 0.f;
+        pacc[i] = 0.f;
+      }
 #pragma unroll
       for (int ks = 0; ks < C::KSTEPS; ks++) {
         const int off = a_row ^ (ks << 5);
-#pragma unroll
-        for (int mi = 0; mi < C::MI; mi++) {
-          const V8 qa = *(const V8*)(q_lds + off + mi * 32 * C::ROWB);
-          const V8 da = *(const V8*)(do_lds + off + mi * 32 * C::ROWB);
-          sacc[mi] = M::mfma32(qa, kf[ks], sacc[mi]);
-          pacc[mi] = M::mfma32(da, vf[ks], pacc[mi]);
-        }
+        const V8 qa = *(const V8*)(q_lds + off + wq * 32 * C::ROWB);
+        const V8 kb = *(const V8*)(k_lds + off);
+        const V8 da = *(const V8*)(do_lds + off + wq * 32 * C::ROWB);
+        const V8 vb = *(const V8*)(v_lds + off);
+        sacc = M::mfma32(qa, kb, sacc);
+        pacc = M::mfma32(da, vb, pacc);
       }
 
       // ---- P and dS -----------------------------------------------------------
-      const bool full = i0 + C::BM - 1 < len_q && jw1 < len_k &&
-                        (a.wr < 0 || jw1 <= i0 + shift + a.wr) &&
-                        (a.wl < 0 || jw0 >= i0 + C::BM - 1 + shift - a.wl || jw1 < a.n_sink);
-      // key position relative to the aligned diagonal of query row i0: rel(i) = rel0 - (i - i0)
-      const int rel0 = jc - i0 - shift;
+      const bool full = iw0 + 31 < len_q && jw1 < len_k &&
+                        (a.wr < 0 || jw1 <= iw0 + shift + a.wr) &&
+                        (a.wl < 0 || jw0 >= iw0 + 31 + shift - a.wl || jw1 < a.n_sink);
+      // key position relative to the aligned diagonal of row iw0: rel(i) = rel0 - (i - iw0)
+      const int rel0 = jc - iw0 - shift;
       const int rel_hi = (a.wr < 0) ? (1 << 30) : a.wr;
       const int rel_lo = (a.wl < 0 || jc < a.n_sink) ? -(1 << 30) : -a.wl;
       const bool col_ok = jc < len_k;
 #pragma unroll
-      for (int mi = 0; mi < C::MI; mi++) {
+      for (int i4 = 0; i4 < 4; i4++) {
+        const int rbase = 8 * i4 + 4 * g;
+        const f32x4 l4 = *(const f32x4*)(lse_lds + rbase);
+        const f32x4 d4 = *(const f32x4*)(delta_lds + rbase);
 #pragma unroll
-        for (int i4 = 0; i4 < 4; i4++) {
-          const int rbase = mi * 32 + 8 * i4 + 4 * g;
-          const f32x4 l4 = *(const f32x4*)(lse_lds + rbase);
-          const f32x4 d4 = *(const f32x4*)(delta_lds + rbase);
-#pragma unroll
-          for (int e = 0; e < 4; e++) {
-            const int i = 4 * i4 + e;
-            float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[mi][i], a.scale_log2, -l4[e]));
-            if (!full) {
-              const int rel = rel0 - (rbase + e);
-              const bool ok = col_ok & (rel <= rel_hi) & (rel >= rel_lo);
-              p = ok ? p : 0.f;  // rows past the end already have lse = +inf
-            }
-            sacc[mi][i] = p;
-            pacc[mi][i] = p * (pacc[mi][i] - d4[e]);
+        for (int e = 0; e < 4; e++) {
+          const int i = 4 * i4 + e;
+          float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[i], a.scale_log2, -l4[e]));
+          if (!full) {
+            const int rel = rel0 - (rbase + e);
+            const bool ok = col_ok & (rel <= rel_hi) & (rel >= rel_lo);
+            p = ok ? p : 0.f;  // rows past the end already have lse = +inf
           }
+          sacc[i] = p;
+          pacc[i] = p * (pacc[i] - d4[e]);
         }
       }
 
       // ---- dV^T += dO^T P ; dK^T += Q^T dS --------------------------------------
 #pragma unroll
-      for (int ks = 0; ks < C::BM / 16; ks++) {
-        const int mi = ks >> 1;
+      for (int ks = 0; ks < 2; ks++) {
         float pv[8], dsv[8];
 #pragma unroll
         for (int j = 0; j < 8; j++) {
-          pv[j] = sacc[mi][8 * (ks & 1) + j];
-          dsv[j] = pacc[mi][8 * (ks & 1) + j];
+          pv[j] = sacc[8 * ks + j];
+          dsv[j] = pacc[8 * ks + j];
         }
         const V8 pb = M::pack(pv);
         const V8 dsb = M::pack(dsv);
+        const int rowoff = (wq * 32 + ks * 16) * C::ROWB;
 #pragma unroll
         for (int d = 0; d < C::DBLK; d++) {
-          const int off0 = (t_row0 ^ (d << 6)) + ks * 16 * C::ROWB;
-          const int off1 = (t_row1 ^ (d << 6)) + ks * 16 * C::ROWB;
+          const int off0 = (t_row0 ^ (d << 6)) + rowoff;
+          const int off1 = (t_row1 ^ (d << 6)) + rowoff;
           dv_acc[d] = M::mfma32(tr_pair<V8>(do_lds + off0, do_lds + off1), pb, dv_acc[d]);
           dk_acc[d] = M::mfma32(tr_pair<V8>(q_lds + off0, q_lds + off1), dsb, dk_acc[d]);
         }
@@ -281,17 +280,37 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
     __syncthreads();
   }
 
-  // ---- write dK, dV (C layout: lane = key, regs = d) ------------------------------
-  if (jc < len_k) {
+  // ---- add the two query halves (through LDS), then write dK, dV --------------------
+  // (C layout: lane = key, regs = d)
+  float* red = (float*)(smem + wk * C::RED_PER_WK);
+  if (wq == 1) {
 #pragma unroll
     for (int d = 0; d < C::DBLK; d++)
 #pragma unroll
       for (int i4 = 0; i4 < 4; i4++) {
+        const f32x4 kk = {dk_acc[d][4 * i4], dk_acc[d][4 * i4 + 1], dk_acc[d][4 * i4 + 2],
+                          dk_acc[d][4 * i4 + 3]};
+        const f32x4 vv = {dv_acc[d][4 * i4], dv_acc[d][4 * i4 + 1], dv_acc[d][4 * i4 + 2],
+                          dv_acc[d][4 * i4 + 3]};
+        *(f32x4*)(red + ((d * 4 + i4) * 64 + lane) * 4) = kk;
+        *(f32x4*)(red + ((C::DBLK * 4 + d * 4 + i4) * 64 + lane) * 4) = vv;
+      }
+  }
+  __syncthreads();
+  if (wq == 0 && jc < len_k) {
+#pragma unroll
+    for (int d = 0; d < C::DBLK; d++)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; i4++) {
+        const f32x4 kk = *(const f32x4*)(red + ((d * 4 + i4) * 64 + lane) * 4);
+        const f32x4 vv = *(const f32x4*)(red + ((C::DBLK * 4 + d * 4 + i4) * 64 + lane) * 4);
         const int col = d * 32 + 8 * i4 + 4 * g;
-        const auto k4 = M::pack4(dk_acc[d][4 * i4] * a.scale, dk_acc[d][4 * i4 + 1] * a.scale,
-                                 dk_acc[d][4 * i4 + 2] * a.scale, dk_acc[d][4 * i4 + 3] * a.scale);
-        const auto v4 = M::pack4(dv_acc[d][4 * i4], dv_acc[d][4 * i4 + 1], dv_acc[d][4 * i4 + 2],
-                                 dv_acc[d][4 * i4 + 3]);
+        const auto k4 = M::pack4((dk_acc[d][4 * i4] + kk[0]) * a.scale,
+                                 (dk_acc[d][4 * i4 + 1] + kk[1]) * a.scale,
+                                 (dk_acc[d][4 * i4 + 2] + kk[2]) * a.scale,
+                                 (dk_acc[d][4 * i4 + 3] + kk[3]) * a.scale);
+        const auto v4 = M::pack4(dv_acc[d][4 * i4] + vv[0], dv_acc[d][4 * i4 + 1] + vv[1],
+                                 dv_acc[d][4 * i4 + 2] + vv[2], dv_acc[d][4 * i4 + 3] + vv[3]);
         *(typename M::V4*)(dk_ptr + (int64_t)jc * a.dk_st[1] + col) = k4;
         *(typename M::V4*)(dv_ptr + (int64_t)jc * a.dv_st[1] + col) = v4;
       }
