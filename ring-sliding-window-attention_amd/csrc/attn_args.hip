@@ -50,6 +50,16 @@ int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a) {
                    rows_aligned(p->v, p->v_stride) && rows_aligned(p->out, p->out_stride),
                RSWA_ERR_UNSUPPORTED, "attn: q/k/v/out rows must start 16-byte aligned");
   RSWA_REQUIRE(((uintptr_t)p->lse) % 4 == 0, RSWA_ERR_UNSUPPORTED, "attn: lse misaligned");
+  {
+    // tiles are fetched through 32-bit buffer offsets relative to a (sequence, head) slice
+    const int64_t rq = packed ? p->total_q : p->seqlen_q, rk = packed ? p->total_k : p->seqlen_k;
+    const int64_t lim = (1ll << 31) - 65536;
+    RSWA_REQUIRE(rq * p->q_stride[1] * 2 < lim && rk * p->k_stride[1] * 2 < lim &&
+                     rk * p->v_stride[1] * 2 < lim && p->q_stride[1] >= 0 &&
+                     p->k_stride[1] >= 0 && p->v_stride[1] >= 0,
+                 RSWA_ERR_UNSUPPORTED,
+                 "attn: one sequence of q, k or v spans 2 GiB or more (rows * row stride)");
+  }
 
   a.q = p->q;
   a.k = p->k;
@@ -101,6 +111,11 @@ int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a) {
     RSWA_REQUIRE(rows_aligned(p->dout, p->dout_stride) && rows_aligned(p->dq, p->dq_stride) &&
                      rows_aligned(p->dk, p->dk_stride) && rows_aligned(p->dv, p->dv_stride),
                  RSWA_ERR_UNSUPPORTED, "attn_bwd: dout/dq/dk/dv rows must start 16-byte aligned");
+    {
+      const int64_t rq = packed ? p->total_q : p->seqlen_q;
+      RSWA_REQUIRE(rq * p->dout_stride[1] * 2 < (1ll << 31) - 65536 && p->dout_stride[1] >= 0,
+                   RSWA_ERR_UNSUPPORTED, "attn_bwd: one sequence of dout spans 2 GiB or more");
+    }
     const uint64_t need = bwd_workspace_bytes(p);
     RSWA_REQUIRE(p->workspace != nullptr || need == 0, RSWA_ERR_INVALID,
                  "attn_bwd: null workspace");

@@ -28,19 +28,6 @@
 namespace rswa {
 namespace {
 
-typedef __attribute__((__vector_size__(8 * sizeof(short)))) short s16x8;
-
-// Two transposing reads -> one 8-element MFMA fragment.
-template <typename V8>
-__device__ __forceinline__ V8 tr_pair(const char* p0, const char* p1) {
-  const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p0);
-  const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p1);
-  const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-  V8 out;
-  __builtin_memcpy(&out, &both, 16);
-  return out;
-}
-
 // ============================================================================
 // dK / dV
 // ============================================================================

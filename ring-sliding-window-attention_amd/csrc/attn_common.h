@@ -161,6 +161,19 @@ __device__ __forceinline__ int swz(int row, int chunk) {
   return chunk ^ swz_f<CH>(row);
 }
 
+typedef __attribute__((__vector_size__(8 * sizeof(short)))) short s16x8;
+
+// Two transposing reads -> one 8-element MFMA fragment.
+template <typename V8>
+__device__ __forceinline__ V8 tr_pair(const char* p0, const char* p1) {
+  const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p0);
+  const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p1);
+  const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  V8 out;
+  __builtin_memcpy(&out, &both, 16);
+  return out;
+}
+
 typedef __attribute__((address_space(3))) void lds_void_t;
 typedef __attribute__((address_space(1))) const void glob_void_t;
 
@@ -188,6 +201,48 @@ __device__ __forceinline__ void g2lds_tile(const T* src, int64_t stride, int val
                                      (lds_void_t*)(lds_tile + slot * 1024), 16, 0, 0);
   }
 }
+
+// Buffer resource over the rows of one (sequence, head) slice: `rows` rows of `row_bytes`
+// useful bytes, `stride_bytes` apart.  Loads past the last row return zero, in registers
+// and in LDS alike, so partial tiles need no clamping.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rows_rsrc(const void* base, int rows,
+                                                                 int64_t stride_bytes,
+                                                                 int row_bytes) {
+  const int64_t bytes = rows > 0 ? (int64_t)(rows - 1) * stride_bytes + row_bytes : 0;
+  return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, (int)bytes, 0x00020000);
+}
+
+// Cooperative copy of a [ROWS x D] tile into a swizzled LDS tile with buffer loads that
+// land directly in LDS (buffer_load_dwordx4 ... lds: lane L of a wave writes
+// wave_base + 16 L).  The per-lane byte offsets are computed once (init); a tile load is
+// then N instructions with one scalar offset and no vector arithmetic at all.
+template <int D, int ROWS, int THREADS>
+struct TileDma {
+  static constexpr int CPR = D / 8;
+  static constexpr int RPI = 64 / CPR;  // rows per wave instruction
+  static constexpr int NW = THREADS / 64;
+  static constexpr int N = ROWS * CPR / THREADS;
+  static_assert(N >= 1 && N * THREADS == ROWS * CPR, "tile must divide evenly");
+  int voff[N];
+  int wave;
+  __device__ __forceinline__ void init(int64_t stride_elems, int tid) {
+    const int lane = tid & 63;
+    wave = tid >> 6;
+#pragma unroll
+    for (int n = 0; n < N; n++) {
+      const int row = (n * NW + wave) * RPI + lane / CPR;
+      voff[n] = (int)(row * stride_elems * 2) + (((lane % CPR) ^ swz_f<CPR>(row)) << 4);
+    }
+  }
+  // `soff` = byte offset of the tile's first row inside the resource (wave-uniform)
+  __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t rsrc, int soff, char* lds_tile) const {
+#pragma unroll
+    for (int n = 0; n < N; n++) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          rsrc, (lds_void_t*)(lds_tile + (n * NW + wave) * 1024), 16, voff[n], soff, 0, 0);
+    }
+  }
+};
 
 // max / sum across the two half-waves (lane l <-> lane l ^ 32).
 __device__ __forceinline__ float halfwave_max(float x) {

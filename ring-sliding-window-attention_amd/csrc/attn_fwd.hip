@@ -3,12 +3,21 @@
 //
 // Replaces flash-attn's forward as wrapped at ring_swa/ops/wrap_flash.py:168-273.
 //
-// One block = 128 query rows of one (sequence, q head); 4 waves x 32 rows.
-// Per 64-key tile a wave computes S^T = K Q^T (keys x queries) with
-// v_mfma_f32_32x32x16, so each lane owns ONE query column: the row max / sum of
-// the online softmax are in-lane reductions plus a single half-wave exchange,
-// and P^T is already laid out as the B operand of O^T += V^T P^T.  V^T fragments
-// come straight out of the row-major V tile with ds_read_b64_tr_b16.
+// One block = 8 waves x 32 query rows sharing every K/V tile it loads: either 128 rows of
+// TWO q heads of one GQA group (group size even) or 256 rows of one q head.  Per 64-key
+// tile a wave computes S^T = K Q^T (keys x queries) with v_mfma_f32_32x32x16, so each
+// lane owns ONE query column: the row max / sum of the online softmax are in-lane
+// reductions plus a single half-wave exchange, and P^T is already laid out as the B
+// operand of O^T += V^T P^T.  V^T fragments come straight out of the row-major V tile
+// with ds_read_b64_tr_b16.
+//
+// Pipeline.  K/V tiles are double-buffered in LDS and filled by buffer loads that land
+// directly in LDS, issued one (V) and two (K) tiles ahead.  The buffers are SEPARATE
+// static __shared__ arrays and the tile loop is unrolled by two, so that every access
+// names its buffer statically: only then can the compiler tell that an in-flight load
+// does not alias the LDS reads of the current tile, and not wait for it.  Inside a wave
+// the loop is software-pipelined: the QK^T MFMAs of tile t+1 are issued together with
+// the softmax (vector ALU) of tile t, so the matrix and vector pipes overlap.
 #include "attn_common.h"
 
 namespace rswa {
@@ -16,33 +25,26 @@ namespace {
 
 template <int D>
 struct FwdCfg {
-  static constexpr int BM = 128;
   static constexpr int BN = 64;
-  static constexpr int THREADS = 256;
+  static constexpr int THREADS = 512;
   static constexpr int KSTEPS = D / 16;
   static constexpr int DBLK = D / 32;
-  static constexpr int CPR = D / 8;  // 16-byte chunks per row
-  static constexpr int CH = BN * CPR / THREADS;
-  // LDS row strides (bytes).  K: +16 B keeps the 16 rows of a b128 phase on distinct
-  // banks.  V: stride = 16 dwords mod 32 so the 4 rows x 64 B of a transposing read
-  // phase cover all 64 banks once.
-  static constexpr int K_STRIDE = D * 2 + 16;
-  static constexpr int V_STRIDE = (D == 128) ? 320 : 192;
-  static constexpr int K_TILE = BN * K_STRIDE;
-  static constexpr int V_TILE = BN * V_STRIDE;
+  static constexpr int CPR = D / 8;   // 16-byte chunks per row
+  static constexpr int ROWB = D * 2;  // bytes per row
+  static constexpr int TILE = BN * ROWB;
   static constexpr int O_STRIDE = D * 2 + 16;
-  static constexpr int SMEM = 2 * K_TILE + 2 * V_TILE;
-  static_assert(SMEM >= 4 * 32 * O_STRIDE, "epilogue staging must fit");
+  static_assert(TILE >= 32 * O_STRIDE, "one wave's epilogue staging fits one tile buffer");
 };
 
 template <typename T, int D>
-// two blocks per CU (2 waves per SIMD): keeps everything in the 256 architectural VGPRs,
-// so no accumulator-register copies, and lets one wave's softmax overlap another's MFMAs
-__global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
+__global__ __launch_bounds__(512) void attn_fwd_kernel(const AttnArgs a) {
   using C = FwdCfg<D>;
   using M = Mma<T>;
   using V8 = typename M::V8;
-  extern __shared__ __attribute__((aligned(16))) char smem[];
+  __shared__ __attribute__((aligned(1024))) char k_s0[C::TILE];
+  __shared__ __attribute__((aligned(1024))) char k_s1[C::TILE];
+  __shared__ __attribute__((aligned(1024))) char v_s0[C::TILE];
+  __shared__ __attribute__((aligned(1024))) char v_s1[C::TILE];
 
   const int wid = logical_block_id(a.n_work);
   if (wid < 0) return;
@@ -51,18 +53,25 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
   const int wave = tid >> 6;
   const int l32 = lane & 31;
   const int g = lane >> 5;
+  const int i16 = lane & 15;
+  const int u = lane >> 4;
 
-  // ---- which (sequence, kv head, q tile, q head) ---------------------------
-  const int hg = wid % a.group;
-  int rest = wid / a.group;
+  // ---- which (sequence, kv head, q tile, q head(s)) -------------------------
+  // pair mode: waves 0-3 and 4-7 take the same 128 rows of two neighbouring q heads;
+  // row mode: the 8 waves take 256 consecutive rows of one q head
+  const bool pair = (a.group & 1) == 0;
+  const int units = pair ? a.group >> 1 : a.group;  // blocks per (kv head, q tile)
+  const int bm = pair ? 128 : 256;                  // query rows per block
+  const int hu = wid % units;
+  int rest = wid / units;
   const int slot = rest % a.n_tile;
   rest /= a.n_tile;
   const int hk = rest % a.heads_kv;
-  const int hq = hk * a.group + hg;
+  const int hq = hk * a.group + (pair ? 2 * hu + (wave >> 2) : hu);
   SeqInfo s;
   int qt;
   if (a.cu_q) {
-    if (!locate_packed(a, slot, C::BM, false, s, qt)) return;
+    if (!locate_packed(a, slot, bm, false, s, qt)) return;
   } else {
     s.batch_idx = rest / a.heads_kv;
     s.q_row0 = s.k_row0 = 0;
@@ -72,7 +81,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
   }
   const int b = s.batch_idx;
   const int len_q = s.len_q, len_k = s.len_k;
-  const int i0 = qt * C::BM;
+  const int i0 = qt * bm;
   if (i0 >= len_q) return;
 
   const T* q_ptr = (const T*)a.q + b * a.q_st[0] + s.q_row0 * a.q_st[1] + hq * a.q_st[2];
@@ -82,7 +91,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
   float* lse_ptr = a.lse + b * a.lse_st[0] + hq * a.lse_st[1] + s.q_row0 * a.lse_st[2];
 
   // ---- key tiles this block visits -----------------------------------------
-  const int i_last = min(i0 + C::BM, len_q) - 1;
+  const int i_last = min(i0 + bm, len_q) - 1;
   const int lo_blk = row_bounds(a, i0, len_q, len_k).lo;
   const int hi_blk = row_bounds(a, i_last, len_q, len_k).hi;
   const bool band = hi_blk >= lo_blk;
@@ -94,10 +103,9 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
   auto tile_of = [&](int it) { return it < n_sink_t ? it : t_lo + (it - n_sink_t); };
 
   // ---- this wave's rows ----------------------------------------------------
-  const int r0 = i0 + wave * 32;
+  const int r0 = i0 + (pair ? wave & 3 : wave) * 32;
   const int iq = r0 + l32;
   const RowBounds rb = row_bounds(a, iq, len_q, len_k);
-  const bool wave_valid = r0 < len_q;
   const bool wave_rows_full = r0 + 31 < len_q;
   const RowBounds wb_first = row_bounds(a, r0, len_q, len_k);
   const RowBounds wb_last = row_bounds(a, min(r0 + 31, len_q - 1), len_q, len_k);
@@ -121,128 +129,151 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
   float m_run = -__builtin_inff();  // running max of raw scores (shared by the lane pair)
   float l_run = 0.f;                // this lane's share of the running sum
 
-  // ---- global -> register -> LDS tile movement ------------------------------
-  u32x4 kreg[C::CH], vreg[C::CH];
-  auto load_tile = [&](int tile) {
-    const int j0 = tile * C::BN;
+  // ---- lane-constant LDS offsets (swizzle folded into XOR / immediate parts) ----
+  // K row fragments (16-byte reads): row = 32 t + l32, chunk = 2 ks + g
+  //   offset = (a_row ^ (ks << 5)) + t * 32 * ROWB
+  const int a_row = l32 * C::ROWB + ((g ^ swz_f<C::CPR>(l32)) << 4);
+  // transposing reads of V: rows 16 s4 + 4 g + (i16 >> 2) and + 8, chunk = 4 d + lp
+  //   offset = (t_row{0,1} ^ (d << 6)) + s4 * 16 * ROWB
+  const int rl = 4 * g + (i16 >> 2);
+  const int lp = 2 * (u & 1) + ((i16 & 3) >> 1);
+  const int t_row0 = rl * C::ROWB + ((lp ^ swz_f<C::CPR>(rl)) << 4) + (i16 & 1) * 8;
+  const int t_row1 = (rl + 8) * C::ROWB + ((lp ^ swz_f<C::CPR>(rl + 8)) << 4) + (i16 & 1) * 8;
+
+  // ---- tile DMA: rows past len_k read as zero ---------------------------------
+  const __amdgpu_buffer_rsrc_t k_rsrc = make_rows_rsrc(k_ptr, len_k, a.k_st[1] * 2, C::ROWB);
+  const __amdgpu_buffer_rsrc_t v_rsrc = make_rows_rsrc(v_ptr, len_k, a.v_st[1] * 2, C::ROWB);
+  TileDma<D, C::BN, C::THREADS> k_dma, v_dma;
+  k_dma.init(a.k_st[1], tid);
+  v_dma.init(a.v_st[1], tid);
+  const int k_tile_bytes = (int)(C::BN * a.k_st[1] * 2), v_tile_bytes = (int)(C::BN * a.v_st[1] * 2);
+  auto load_k = [&](int it, char* dst) __attribute__((always_inline)) {
+    k_dma.load(k_rsrc, tile_of(it) * k_tile_bytes, dst);
+  };
+  auto load_v = [&](int it, char* dst) __attribute__((always_inline)) {
+    v_dma.load(v_rsrc, tile_of(it) * v_tile_bytes, dst);
+  };
+
+  // ---- pieces of one tile ------------------------------------------------------
+  // S^T[key, query] = K Q^T
+  auto qk = [&](const char* kc, f32x16(&sacc)[2]) __attribute__((always_inline)) {
 #pragma unroll
-    for (int n = 0; n < C::CH; n++) {
-      const int c = tid + n * C::THREADS;
-      const int row = c / C::CPR, col = (c % C::CPR) * 8;
-      if (j0 + row < len_k) {
-        kreg[n] = *(const u32x4*)(k_ptr + (int64_t)(j0 + row) * a.k_st[1] + col);
-        vreg[n] = *(const u32x4*)(v_ptr + (int64_t)(j0 + row) * a.v_st[1] + col);
-      } else {
-        kreg[n] = u32x4{0, 0, 0, 0};
-        vreg[n] = u32x4{0, 0, 0, 0};
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) sacc[t][i] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < C::KSTEPS; ks++) {
+      const int off = a_row ^ (ks << 5);
+#pragma unroll
+      for (int t = 0; t < 2; t++) {
+        const V8 kf = *(const V8*)(kc + off + t * 32 * C::ROWB);
+        sacc[t] = M::mfma32(kf, qf[ks], sacc[t]);
       }
     }
   };
-  auto store_tile = [&](int buf) {
-#pragma unroll
-    for (int n = 0; n < C::CH; n++) {
-      const int c = tid + n * C::THREADS;
-      const int row = c / C::CPR, col = (c % C::CPR) * 8;
-      *(u32x4*)(smem + buf * C::K_TILE + row * C::K_STRIDE + col * 2) = kreg[n];
-      *(u32x4*)(smem + 2 * C::K_TILE + buf * C::V_TILE + row * C::V_STRIDE + col * 2) = vreg[n];
-    }
-  };
-
-  if (n_tiles > 0) {
-    load_tile(tile_of(0));
-    store_tile(0);
-  }
-  __syncthreads();
-
-  for (int it = 0; it < n_tiles; it++) {
-    const int buf = it & 1;
+  // mask of an edge tile: visible iff j <= hi and (j >= lo or j < n_sink)
+  auto mask = [&](int it, f32x16(&sacc)[2]) __attribute__((always_inline)) {
     const int j0 = tile_of(it) * C::BN;
     const int j1 = j0 + C::BN - 1;
-    if (it + 1 < n_tiles) load_tile(tile_of(it + 1));
-
-    const bool needed =
-        wave_valid && j0 <= wb_last.hi && (j1 >= wb_first.lo || j0 < a.n_sink);
-    if (needed) {
-      const char* kbuf = smem + buf * C::K_TILE;
-      const char* vbuf = smem + 2 * C::K_TILE + buf * C::V_TILE;
-      // S^T[key, query] = K Q^T
-      f32x16 sacc[2];
-#pragma unroll
-      for (int t = 0; t < 2; t++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) sacc[t][i] = 0.f;
-#pragma unroll
-      for (int ks = 0; ks < C::KSTEPS; ks++) {
-#pragma unroll
-        for (int t = 0; t < 2; t++) {
-          const V8 kf = *(const V8*)(kbuf + (t * 32 + l32) * C::K_STRIDE + (ks * 16 + g * 8) * 2);
-          sacc[t] = M::mfma32(kf, qf[ks], sacc[t]);
-        }
-      }
-      const bool full = wave_rows_full && j1 <= wb_first.hi &&
-                        (j0 >= wb_last.lo || j1 < a.n_sink);
-      if (!full) {
-#pragma unroll
-        for (int t = 0; t < 2; t++)
-#pragma unroll
-          for (int i = 0; i < 16; i++) {
-            const int j = j0 + t * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
-            const bool ok = j <= rb.hi && (j >= rb.lo || j < a.n_sink);
-            sacc[t][i] = ok ? sacc[t][i] : -__builtin_inff();
-          }
-      }
-      // online softmax (raw-score max; exponent in base 2)
-      float mx = sacc[0][0];
-#pragma unroll
-      for (int t = 0; t < 2; t++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) mx = fmaxf(mx, sacc[t][i]);
-      mx = halfwave_max(mx);
-      const float m_new = fmaxf(m_run, mx);
-      const float m_use = (m_new == -__builtin_inff()) ? 0.f : m_new;
-      const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * a.scale_log2);
-      const float mc = m_use * a.scale_log2;
-      m_run = m_new;
-      float psum = 0.f;
+    const bool full =
+        wave_rows_full && j1 <= wb_first.hi && (j0 >= wb_last.lo || j1 < a.n_sink);
+    if (!full) {
+      const int hi_rel = rb.hi - j0;
+      const int lo_rel = rb.lo - j0;
+      const int sink_rel = a.n_sink - j0;
 #pragma unroll
       for (int t = 0; t < 2; t++)
 #pragma unroll
         for (int i = 0; i < 16; i++) {
-          const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[t][i], a.scale_log2, -mc));
-          sacc[t][i] = p;
-          psum += p;
+          const int j = t * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
+          const bool ok = (j <= hi_rel) & ((j >= lo_rel) | (j < sink_rel));
+          sacc[t][i] = ok ? sacc[t][i] : -__builtin_inff();
         }
-      l_run = l_run * alpha + psum;
-      if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {
+    }
+  };
+  // online softmax of one tile (raw-score max, exponent in base 2); P^T packed for the
+  // PV MFMAs; returns the factor the running output must be scaled by
+  auto softmax = [&](f32x16(&sacc)[2], V8(&pb)[4]) __attribute__((always_inline)) -> float {
+    float mx = sacc[0][0];
 #pragma unroll
-        for (int d = 0; d < C::DBLK; d++)
+    for (int t = 0; t < 2; t++)
 #pragma unroll
-          for (int i = 0; i < 16; i++) o_acc[d][i] *= alpha;
+      for (int i = 0; i < 16; i++) mx = fmaxf(mx, sacc[t][i]);
+    mx = halfwave_max(mx);
+    const float m_new = fmaxf(m_run, mx);
+    const float m_use = (m_new == -__builtin_inff()) ? 0.f : m_new;
+    const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * a.scale_log2);
+    const float mc = m_use * a.scale_log2;
+    m_run = m_new;
+    float psum = 0.f;
+#pragma unroll
+    for (int s4 = 0; s4 < 4; s4++) {
+      float pv[8];
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        pv[j] = __builtin_amdgcn_exp2f(
+            __builtin_fmaf(sacc[s4 >> 1][8 * (s4 & 1) + j], a.scale_log2, -mc));
+        psum += pv[j];
       }
-      // O^T[d, query] += V^T P^T
-      const int i16 = lane & 15, u = lane >> 4;
-      const char* vlane = vbuf + (4 * g + (i16 >> 2)) * C::V_STRIDE + (16 * (u & 1) + 4 * (i16 & 3)) * 2;
+      pb[s4] = M::pack(pv);
+    }
+    l_run = l_run * alpha + psum;
+    return alpha;
+  };
+  // O^T[d, query] = alpha * O^T + V^T P^T
+  auto pv_acc = [&](const char* vc, const V8(&pb)[4], float alpha) __attribute__((always_inline)) {
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {
 #pragma unroll
-      for (int s4 = 0; s4 < 4; s4++) {
-        float pv[8];
+      for (int d = 0; d < C::DBLK; d++)
 #pragma unroll
-        for (int j = 0; j < 8; j++) pv[j] = sacc[s4 >> 1][8 * (s4 & 1) + j];
-        const V8 pb = M::pack(pv);
+        for (int i = 0; i < 16; i++) o_acc[d][i] *= alpha;
+    }
 #pragma unroll
-        for (int d = 0; d < C::DBLK; d++) {
-          const char* p0 = vlane + (s4 * 16) * C::V_STRIDE + d * 64;
-          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p0);
-          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p0 + 8 * C::V_STRIDE));
-          typedef __attribute__((__vector_size__(8 * sizeof(short)))) short s16x8;
-          const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-          V8 vf;
-          __builtin_memcpy(&vf, &both, 16);
-          o_acc[d] = M::mfma32(vf, pb, o_acc[d]);
-        }
+    for (int s4 = 0; s4 < 4; s4++) {
+#pragma unroll
+      for (int d = 0; d < C::DBLK; d++) {
+        const int off0 = (t_row0 ^ (d << 6)) + s4 * 16 * C::ROWB;
+        const int off1 = (t_row1 ^ (d << 6)) + s4 * 16 * C::ROWB;
+        o_acc[d] = M::mfma32(tr_pair<V8>(vc + off0, vc + off1), pb[s4], o_acc[d]);
       }
     }
-    if (it + 1 < n_tiles) store_tile(buf ^ 1);
+  };
+
+  // ---- pipelined tile loop ----------------------------------------------------------
+  // entering step(t): S(t) is in s_cur; K(t+1) and V(t) are in LDS (kn, vc); the buffer kc
+  // that held K(t) is free.  The step starts the loads of K(t+2) -> kc and V(t+1) -> vn,
+  // computes S(t+1) under the softmax of tile t, accumulates P(t) V(t), and syncs.
+  f32x16 s_cur[2], s_nxt[2];
+  auto step = [&](int it, char* kc, const char* kn, const char* vc,
+                  char* vn) __attribute__((always_inline)) {
+    if (it + 2 < n_tiles) load_k(it + 2, kc);
+    if (it + 1 < n_tiles) load_v(it + 1, vn);
+    mask(it, s_cur);
+    V8 pb[4];
+    float alpha;
+    if (it + 1 < n_tiles) {
+      qk(kn, s_nxt);
+      alpha = softmax(s_cur, pb);
+    } else {
+      alpha = softmax(s_cur, pb);
+    }
+    pv_acc(vc, pb, alpha);
+#pragma unroll
+    for (int t = 0; t < 2; t++) s_cur[t] = s_nxt[t];
     __syncthreads();
+  };
+
+  if (n_tiles > 0) {
+    load_k(0, k_s0);
+    load_v(0, v_s0);
+  }
+  if (n_tiles > 1) load_k(1, k_s1);
+  __syncthreads();
+  if (n_tiles > 0) qk(k_s0, s_cur);
+  __syncthreads();  // every wave has read K(0) before step(0) overwrites its buffer
+  for (int it = 0; it < n_tiles; it += 2) {
+    step(it, k_s0, k_s1, v_s0, v_s1);
+    if (it + 1 < n_tiles) step(it + 1, k_s1, k_s0, v_s1, v_s0);
   }
 
   // ---- epilogue --------------------------------------------------------------
@@ -252,48 +283,59 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
     lse_ptr[(int64_t)iq * a.lse_st[2]] =
         l_tot > 0.f ? m_run * a.scale + __logf(l_tot) : -__builtin_inff();
   }
-  // transpose O^T through LDS (per-wave region) for coalesced 16-byte stores
-  char* stage = smem + wave * 32 * C::O_STRIDE;
+  // transpose O^T through LDS for coalesced 16-byte stores: waves 0-3 first (one tile
+  // buffer each), then waves 4-7
+  char* stage = (wave & 3) == 0 ? k_s0 : (wave & 3) == 1 ? k_s1 : (wave & 3) == 2 ? v_s0 : v_s1;
+  for (int half = 0; half < 2; half++) {
+    if ((wave >> 2) == half) {
 #pragma unroll
-  for (int d = 0; d < C::DBLK; d++)
+      for (int d = 0; d < C::DBLK; d++)
 #pragma unroll
-    for (int i4 = 0; i4 < 4; i4++) {
-      const auto h4 = M::pack4(o_acc[d][4 * i4] * inv, o_acc[d][4 * i4 + 1] * inv,
-                               o_acc[d][4 * i4 + 2] * inv, o_acc[d][4 * i4 + 3] * inv);
-      *(typename M::V4*)(stage + l32 * C::O_STRIDE + (d * 32 + 8 * i4 + 4 * g) * 2) = h4;
+        for (int i4 = 0; i4 < 4; i4++) {
+          const auto h4 = M::pack4(o_acc[d][4 * i4] * inv, o_acc[d][4 * i4 + 1] * inv,
+                                   o_acc[d][4 * i4 + 2] * inv, o_acc[d][4 * i4 + 3] * inv);
+          *(typename M::V4*)(stage + l32 * C::O_STRIDE + (d * 32 + 8 * i4 + 4 * g) * 2) = h4;
+        }
     }
-  __syncthreads();
+    __syncthreads();
+    if ((wave >> 2) == half) {
 #pragma unroll
-  for (int n = 0; n < 32 * C::CPR / 64; n++) {
-    const int c = lane + n * 64;
-    const int row = c / C::CPR, col = (c % C::CPR) * 8;
-    if (r0 + row < len_q) {
-      const u32x4 val = *(const u32x4*)(stage + row * C::O_STRIDE + col * 2);
-      *(u32x4*)(o_ptr + (int64_t)(r0 + row) * a.o_st[1] + col) = val;
+      for (int n = 0; n < 32 * C::CPR / 64; n++) {
+        const int c = lane + n * 64;
+        const int row = c / C::CPR, col = (c % C::CPR) * 8;
+        if (r0 + row < len_q) {
+          const u32x4 val = *(const u32x4*)(stage + row * C::O_STRIDE + col * 2);
+          *(u32x4*)(o_ptr + (int64_t)(r0 + row) * a.o_st[1] + col) = val;
+        }
+      }
     }
+    __syncthreads();
   }
 }
+
+// Explicit instantiations: with implicit instantiation alone this hipcc emits the host
+// launch stubs of only some of the four variants.
+template __global__ void attn_fwd_kernel<__bf16, 128>(const AttnArgs);
+template __global__ void attn_fwd_kernel<__bf16, 64>(const AttnArgs);
+template __global__ void attn_fwd_kernel<_Float16, 128>(const AttnArgs);
+template __global__ void attn_fwd_kernel<_Float16, 64>(const AttnArgs);
 
 template <typename T, int D>
 int launch_fwd(AttnArgs& a, hipStream_t stream) {
   using C = FwdCfg<D>;
+  const bool pair = (a.group & 1) == 0;
+  const int bm = pair ? 128 : 256;
+  const int units = (pair ? a.group / 2 : a.group) * a.heads_kv;  // blocks per q tile
   if (a.cu_q) {
-    a.n_tile = (int)(ceil_div(a.rows_q, C::BM) + a.batch);
-    a.n_work = a.n_tile * a.heads_q;
+    a.n_tile = (int)(ceil_div(a.rows_q, bm) + a.batch);
+    a.n_work = a.n_tile * units;
   } else {
-    a.n_tile = (int)ceil_div(a.seqlen_q, C::BM);
-    a.n_work = a.n_tile * a.heads_q * a.batch;
+    a.n_tile = (int)ceil_div(a.seqlen_q, bm);
+    a.n_work = a.n_tile * units * a.batch;
   }
   if (a.n_work == 0) return RSWA_OK;
-  auto kern = attn_fwd_kernel<T, D>;
-  static bool configured = false;  // benign race: the attribute call is idempotent
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       C::SMEM);
-    if (e != hipSuccess) return fail(RSWA_ERR_LAUNCH, "attn_fwd: set smem: %s", hipGetErrorString(e));
-    configured = true;
-  }
-  hipLaunchKernelGGL(kern, dim3(padded_grid(a.n_work)), dim3(C::THREADS), C::SMEM, stream, a);
+  hipLaunchKernelGGL((attn_fwd_kernel<T, D>), dim3(padded_grid(a.n_work)), dim3(C::THREADS), 0,
+                     stream, a);
   return check_launch("attn_fwd");
 }
 
