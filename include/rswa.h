@@ -160,8 +160,8 @@ int rswa_attn_fwd(const rswa_attn_params* p, void* stream);
 int rswa_attn_bwd(const rswa_attn_params* p, void* stream);
 
 /*
- * rswa_attn_bwd is three launches: PREP (delta = rowsum(dout * out) into the
- * workspace), DKDV (dk, dv written; reads delta) and DQ (dq written; reads delta).
+ * rswa_attn_bwd is three launches: PREP (row statistics into the workspace), DKDV
+ * (dk, dv written; reads the statistics) and DQ (dq written; reads the statistics).
  * This variant enqueues only the phases named in the bit mask, on the same
  * workspace: it lets a profiler or benchmark bracket one kernel alone, and lets a
  * caller that needs only some of the gradients skip the rest.  Same interface
@@ -172,7 +172,8 @@ int rswa_attn_bwd(const rswa_attn_params* p, void* stream);
 #define RSWA_BWD_DQ 4
 int rswa_attn_bwd_phases(const rswa_attn_params* p, void* stream, int phases);
 
-/* Scratch rswa_attn_bwd needs for these shapes (fp32 row sums of dout * out). */
+/* Scratch rswa_attn_bwd needs for these shapes: two fp32 values per (row, q head) —
+ * the row sum of dout * out and the LSE in base-2 units. */
 uint64_t rswa_attn_bwd_workspace_bytes(const rswa_attn_params* p);
 
 /* Message of the calling thread's last failed call ("" if none). */

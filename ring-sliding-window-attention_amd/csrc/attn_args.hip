@@ -13,7 +13,7 @@ static uint64_t delta_bytes(const rswa_attn_params* p) {
 
 uint64_t bwd_workspace_bytes(const rswa_attn_params* p) {
   if (!p || p->batch <= 0 || p->heads_q <= 0 || p->head_dim <= 0) return 0;
-  return delta_bytes(p);
+  return 2 * delta_bytes(p);
 }
 
 static bool rows_aligned(const void* ptr, const int64_t* st) {
@@ -71,6 +71,7 @@ int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a) {
   a.dk = p->dk;
   a.dv = p->dv;
   a.delta = nullptr;
+  a.lse2 = nullptr;
   a.cu_q = p->cu_seqlens_q;
   a.cu_k = p->cu_seqlens_k;
   for (int i = 0; i < 3; i++) {
@@ -124,7 +125,10 @@ int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a) {
                  (unsigned long long)p->workspace_bytes, (unsigned long long)need);
     RSWA_REQUIRE(((uintptr_t)p->workspace) % 256 == 0, RSWA_ERR_INVALID,
                  "attn_bwd: workspace must be 256-byte aligned");
-    a.delta = (float*)p->workspace;
+    a.lse2 = (float*)p->workspace;
+    a.delta = (float*)((char*)p->workspace + delta_bytes(p));
+    RSWA_REQUIRE(2 * delta_bytes(p) < (1ull << 31), RSWA_ERR_UNSUPPORTED,
+                 "attn_bwd: rows * heads_q too large for the statistics workspace");
   }
   return RSWA_OK;
 }

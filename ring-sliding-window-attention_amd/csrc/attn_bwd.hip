@@ -2,14 +2,16 @@
 //
 // Replaces flash-attn's backward as wrapped at ring_swa/ops/wrap_flash.py:276-429.
 // Three launches on the caller's stream:
-//   PREP : delta[h][row] = sum_d dO * O   (fp32, in the caller's workspace)
+//   PREP : per (row, q head): delta = sum_d dO * O and lse2 = lse * log2(e) (-inf -> +inf),
+//          both fp32, into the caller's workspace
 //   DKDV : one block (8 waves) owns 128 keys of one (sequence, kv head), keeps their K and
 //          V tiles in LDS and walks the query tiles (64 rows) that can see them, for every
 //          q head of the GQA group; wave (wk, wq) handles key columns 32 wk.. of query rows
 //          32 wq.. of each tile; dK^T / dV^T partials stay in registers for the whole walk,
 //          the two query halves are added through LDS at the end and written once
-//   DQ   : one block owns 128 queries of one (sequence, q head) and walks the key tiles
-//          (64 keys) it can see, like the forward kernel; dQ^T stays in registers
+//   DQ   : one block (8 waves x 32 query rows: 128 rows of two q heads of a GQA group, or
+//          256 rows of one head) walks the key tiles (64 keys) it can see, like the forward
+//          kernel; dQ^T stays in registers
 // S and dP are computed in both main kernels (7 GEMM units instead of 5).  That costs
 // less here than fp32 atomics on dQ: the L2 retires about one fp32 atomic per clock per
 // channel, which caps an atomic dQ far below the MFMA rate.  It also makes the result
@@ -17,12 +19,16 @@
 //
 // DKDV per (query half-tile, wave) (C layout: lane = key):
 //   S = Q K^T, dP = dO V^T      A = Q / dO row fragments, B = K / V row fragments (all LDS)
-//   P = exp2(S*c - lse*log2e), dS = P * (dP - delta)
+//   P = exp2(S*c - lse2), dS = P * (dP - delta)
 //   dV^T += dO^T P, dK^T += Q^T dS   A = transposing LDS reads of dO / Q, B = P / dS (regs)
-// DQ per (key tile, wave); wave w owns query columns 32w..32w+31 (C layout: lane = query):
+// DQ per (key tile, wave); wave owns 32 query columns (C layout: lane = query):
 //   S^T = K Q^T, dP^T = V dO^T  A = K / V row fragments from LDS, B = Q / dO fragments (regs)
-//   dS^T as above with per-lane lse / delta
+//   dS^T as above with per-lane lse2 / delta
 //   dQ^T += K^T dS^T            A = transposing LDS reads of K, B = dS^T (regs)
+//
+// Tiles are double-buffered in SEPARATE static __shared__ arrays, filled by buffer loads
+// that land directly in LDS one tile ahead, and the tile loops are unrolled by two so that
+// every access names its buffer statically (see attn_fwd.hip for why).
 #include "attn_common.h"
 
 namespace rswa {
@@ -33,8 +39,8 @@ namespace {
 // ============================================================================
 template <int D>
 struct DkvCfg {
-  static constexpr int BM = 64;   // query rows per step
-  static constexpr int BN = 128;  // keys per block
+  static constexpr int BM = 64;        // query rows per step
+  static constexpr int BN = 128;       // keys per block
   static constexpr int THREADS = 512;  // 8 waves: 4 key groups x 2 query halves
   static constexpr int KSTEPS = D / 16;
   static constexpr int DBLK = D / 32;
@@ -42,16 +48,11 @@ struct DkvCfg {
   static constexpr int ROWB = D * 2;  // bytes per row
   static constexpr int Q_TILE = BM * ROWB;
   static constexpr int KV_TILE = BN * ROWB;
-  static constexpr int OFF_K = 0;
-  static constexpr int OFF_V = KV_TILE;
-  static constexpr int OFF_Q = 2 * KV_TILE;            // 2 buffers
-  static constexpr int OFF_DO = OFF_Q + 2 * Q_TILE;    // 2 buffers
-  static constexpr int OFF_ST = OFF_DO + 2 * Q_TILE;   // lse2[2][BM], delta[2][BM] fp32
-  static constexpr int SMEM = OFF_ST + 4 * BM * 4;
-  // end-of-walk reduction of the two query halves: per key group 2 matrices of
-  // DBLK x 16 registers x 64 lanes fp32
-  static constexpr int RED_PER_WK = 2 * DBLK * 16 * 64 * 4;
-  static_assert(4 * RED_PER_WK <= SMEM, "reduction staging must fit");
+  // end-of-walk reduction of the two query halves, one matrix (dK, then dV) at a time:
+  // per key group DBLK x 16 registers x 64 lanes fp32, staged in the K tile (key groups
+  // 0-1) and the V tile (key groups 2-3)
+  static constexpr int RED_PER_WK = DBLK * 16 * 64 * 4;
+  static_assert(2 * RED_PER_WK <= KV_TILE, "reduction staging must fit the K and V tiles");
 };
 
 template <typename T, int D>
@@ -59,7 +60,14 @@ __global__ __launch_bounds__(512) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   using C = DkvCfg<D>;
   using M = Mma<T>;
   using V8 = typename M::V8;
-  extern __shared__ __attribute__((aligned(16))) char smem[];
+  __shared__ __attribute__((aligned(1024))) char k_s[C::KV_TILE];
+  __shared__ __attribute__((aligned(1024))) char v_s[C::KV_TILE];
+  __shared__ __attribute__((aligned(1024))) char q_s0[C::Q_TILE];
+  __shared__ __attribute__((aligned(1024))) char q_s1[C::Q_TILE];
+  __shared__ __attribute__((aligned(1024))) char do_s0[C::Q_TILE];
+  __shared__ __attribute__((aligned(1024))) char do_s1[C::Q_TILE];
+  __shared__ __attribute__((aligned(1024))) float st_s0[2 * C::BM];  // lse2[BM], delta[BM]
+  __shared__ __attribute__((aligned(1024))) float st_s1[2 * C::BM];
 
   const int wid = logical_block_id(a.n_work);
   if (wid < 0) return;
@@ -95,8 +103,8 @@ __global__ __launch_bounds__(512) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   const int j_last = min(j0 + C::BN, len_k) - 1;
   const int shift = a.shift_explicit ? a.shift_val : len_k - len_q;
 
-  const T* k_ptr = (const T*)a.k + b * a.k_st[0] + (s.k_row0 + j0) * a.k_st[1] + hk * a.k_st[2];
-  const T* v_ptr = (const T*)a.v + b * a.v_st[0] + (s.k_row0 + j0) * a.v_st[1] + hk * a.v_st[2];
+  const T* k_ptr = (const T*)a.k + b * a.k_st[0] + s.k_row0 * a.k_st[1] + hk * a.k_st[2];
+  const T* v_ptr = (const T*)a.v + b * a.v_st[0] + s.k_row0 * a.v_st[1] + hk * a.v_st[2];
   T* dk_ptr = (T*)a.dk + b * a.dk_st[0] + s.k_row0 * a.dk_st[1] + hk * a.dk_st[2];
   T* dv_ptr = (T*)a.dv + b * a.dv_st[0] + s.k_row0 * a.dv_st[1] + hk * a.dv_st[2];
   const int64_t ws_row0 = a.cu_q ? s.q_row0 : (int64_t)b * a.seqlen_q;
@@ -132,59 +140,62 @@ __global__ __launch_bounds__(512) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   const int t_row0 = rl * C::ROWB + ((lp ^ swz_f<C::CPR>(rl)) << 4) + (i16 & 1) * 8;
   const int t_row1 = (rl + 8) * C::ROWB + ((lp ^ swz_f<C::CPR>(rl + 8)) << 4) + (i16 & 1) * 8;
 
-  // ---- tile movement: everything lands in LDS directly; lse, delta via one register ----
-  float streg = 0.f;
-  auto iter_coords = [&](int it, int& hq, int& i0) {
+  // ---- tile DMA (rows past the end of the sequence read as zero) ------------------
+  TileDma<D, C::BN, C::THREADS> k_dma, v_dma;
+  TileDma<D, C::BM, C::THREADS> q_dma, do_dma;
+  k_dma.init(a.k_st[1], tid);
+  v_dma.init(a.v_st[1], tid);
+  q_dma.init(a.q_st[1], tid);
+  do_dma.init(a.do_st[1], tid);
+  const T* q_base = (const T*)a.q + b * a.q_st[0] + s.q_row0 * a.q_st[1];
+  const T* do_base = (const T*)a.dout + b * a.do_st[0] + s.q_row0 * a.do_st[1];
+  // statistics: one resource over both workspace arrays (lse2 then delta); rows past the
+  // sequence end read a neighbour's finite values, which the row mask / zero Q, dO rows void
+  const int64_t stat_elems = a.delta - a.lse2;  // elements between the two arrays
+  const __amdgpu_buffer_rsrc_t st_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)a.lse2, 0, (int)((stat_elems + a.heads_q * a.rows_q) * 4), 0x00020000);
+
+  auto iter_coords = [&](int it, int& hq, int& i0) __attribute__((always_inline)) {
     hq = hk * a.group + it / n_qt;
     i0 = (qt_lo + it % n_qt) * C::BM;
   };
-  auto load_iter = [&](int it, int buf) {
+  auto load_iter = [&](int it, char* qd, char* dod, float* std_) __attribute__((always_inline)) {
     int hq, i0;
     iter_coords(it, hq, i0);
-    const T* q_ptr = (const T*)a.q + b * a.q_st[0] + (s.q_row0 + i0) * a.q_st[1] + hq * a.q_st[2];
-    const T* do_ptr =
-        (const T*)a.dout + b * a.do_st[0] + (s.q_row0 + i0) * a.do_st[1] + hq * a.do_st[2];
-    g2lds_tile<T, D, C::BM, C::THREADS>(q_ptr, a.q_st[1], len_q - i0,
-                                         smem + C::OFF_Q + buf * C::Q_TILE, tid);
-    g2lds_tile<T, D, C::BM, C::THREADS>(do_ptr, a.do_st[1], len_q - i0,
-                                         smem + C::OFF_DO + buf * C::Q_TILE, tid);
-    if (tid < C::BM) {
-      // lse in base-2 units; rows that must contribute nothing get +inf (P = 0)
-      const int i = i0 + tid;
-      float l = __builtin_inff();
-      if (i < len_q) {
-        l = a.lse[b * a.lse_st[0] + hq * a.lse_st[1] + (s.q_row0 + i) * a.lse_st[2]];
-        l = (l == -__builtin_inff()) ? __builtin_inff() : l * kLog2e;
-      }
-      streg = l;
-    } else if (tid < 2 * C::BM) {
-      const int i = i0 + tid - C::BM;
-      streg = (i < len_q) ? a.delta[(int64_t)hq * a.rows_q + ws_row0 + i] : 0.f;
+    const __amdgpu_buffer_rsrc_t q_rsrc =
+        make_rows_rsrc(q_base + hq * a.q_st[2], len_q, a.q_st[1] * 2, C::ROWB);
+    const __amdgpu_buffer_rsrc_t do_rsrc =
+        make_rows_rsrc(do_base + hq * a.do_st[2], len_q, a.do_st[1] * 2, C::ROWB);
+    q_dma.load(q_rsrc, (int)(i0 * a.q_st[1] * 2), qd);
+    do_dma.load(do_rsrc, (int)(i0 * a.do_st[1] * 2), dod);
+    if (wave < 2) {  // wave 0: lse2 tile, wave 1: delta tile (64 floats each)
+      const int soff = (int)(((int64_t)hq * a.rows_q + ws_row0 + i0 + wave * stat_elems) * 4);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(st_rsrc, (lds_void_t*)(std_ + wave * C::BM), 4,
+                                               lane * 4, soff, 0, 0);
     }
-  };
-  auto store_stats = [&](int buf) {
-    if (tid < 2 * C::BM) *(float*)(smem + C::OFF_ST + buf * 2 * C::BM * 4 + tid * 4) = streg;
   };
 
   if (n_iter > 0) {
-    g2lds_tile<T, D, C::BN, C::THREADS>(k_ptr, a.k_st[1], len_k - j0, smem + C::OFF_K, tid);
-    g2lds_tile<T, D, C::BN, C::THREADS>(v_ptr, a.v_st[1], len_k - j0, smem + C::OFF_V, tid);
-    load_iter(0, 0);
-    store_stats(0);
+    const __amdgpu_buffer_rsrc_t k_rsrc = make_rows_rsrc(k_ptr, len_k, a.k_st[1] * 2, C::ROWB);
+    const __amdgpu_buffer_rsrc_t v_rsrc = make_rows_rsrc(v_ptr, len_k, a.v_st[1] * 2, C::ROWB);
+    k_dma.load(k_rsrc, (int)(j0 * a.k_st[1] * 2), k_s);
+    v_dma.load(v_rsrc, (int)(j0 * a.v_st[1] * 2), v_s);
+    load_iter(0, q_s0, do_s0, st_s0);
   }
   __syncthreads();
 
-  const char* k_lds = smem + C::OFF_K + wk * 32 * C::ROWB;
-  const char* v_lds = smem + C::OFF_V + wk * 32 * C::ROWB;
+  const char* k_lds = k_s + wk * 32 * C::ROWB;
+  const char* v_lds = v_s + wk * 32 * C::ROWB;
 
-  for (int it = 0; it < n_iter; it++) {
-    const int buf = it & 1;
+  // one query tile: prefetch the next one into (qn, don, stn), compute on (qc, doc, stc)
+  auto step = [&](int it, const char* qc, const char* doc, const float* stc, char* qn, char* don,
+                  float* stn) __attribute__((always_inline)) {
     int hq, i0;
     iter_coords(it, hq, i0);
-    if (it + 1 < n_iter) load_iter(it + 1, buf ^ 1);
-    const char* q_lds = smem + C::OFF_Q + buf * C::Q_TILE;
-    const char* do_lds = smem + C::OFF_DO + buf * C::Q_TILE;
-    const float* lse_lds = (const float*)(smem + C::OFF_ST + buf * 2 * C::BM * 4) + wq * 32;
+    if (it + 1 < n_iter) load_iter(it + 1, qn, don, stn);
+    const char* q_lds = qc + wq * 32 * C::ROWB;
+    const char* do_lds = doc + wq * 32 * C::ROWB;
+    const float* lse_lds = stc + wq * 32;
     const float* delta_lds = lse_lds + C::BM;
 
     // Does any (query of this wave's half-tile, key of this wave) pair survive the mask?
@@ -205,9 +216,9 @@ __global__ __launch_bounds__(512) void attn_bwd_dkdv_kernel(const AttnArgs a) {
 #pragma unroll
       for (int ks = 0; ks < C::KSTEPS; ks++) {
         const int off = a_row ^ (ks << 5);
-        const V8 qa = *(const V8*)(q_lds + off + wq * 32 * C::ROWB);
+        const V8 qa = *(const V8*)(q_lds + off);
         const V8 kb = *(const V8*)(k_lds + off);
-        const V8 da = *(const V8*)(do_lds + off + wq * 32 * C::ROWB);
+        const V8 da = *(const V8*)(do_lds + off);
         const V8 vb = *(const V8*)(v_lds + off);
         sacc = M::mfma32(qa, kb, sacc);
         pacc = M::mfma32(da, vb, pacc);
@@ -217,27 +228,42 @@ __global__ __launch_bounds__(512) void attn_bwd_dkdv_kernel(const AttnArgs a) {
       const bool full = iw0 + 31 < len_q && jw1 < len_k &&
                         (a.wr < 0 || jw1 <= iw0 + shift + a.wr) &&
                         (a.wl < 0 || jw0 >= iw0 + 31 + shift - a.wl || jw1 < a.n_sink);
-      // key position relative to the aligned diagonal of row iw0: rel(i) = rel0 - (i - iw0)
-      const int rel0 = jc - iw0 - shift;
-      const int rel_hi = (a.wr < 0) ? (1 << 30) : a.wr;
-      const int rel_lo = (a.wl < 0 || jc < a.n_sink) ? -(1 << 30) : -a.wl;
-      const bool col_ok = jc < len_k;
+      if (full) {
 #pragma unroll
-      for (int i4 = 0; i4 < 4; i4++) {
-        const int rbase = 8 * i4 + 4 * g;
-        const f32x4 l4 = *(const f32x4*)(lse_lds + rbase);
-        const f32x4 d4 = *(const f32x4*)(delta_lds + rbase);
+        for (int i4 = 0; i4 < 4; i4++) {
+          const int rbase = 8 * i4 + 4 * g;
+          const f32x4 l4 = *(const f32x4*)(lse_lds + rbase);
+          const f32x4 d4 = *(const f32x4*)(delta_lds + rbase);
 #pragma unroll
-        for (int e = 0; e < 4; e++) {
-          const int i = 4 * i4 + e;
-          float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[i], a.scale_log2, -l4[e]));
-          if (!full) {
-            const int rel = rel0 - (rbase + e);
-            const bool ok = col_ok & (rel <= rel_hi) & (rel >= rel_lo);
-            p = ok ? p : 0.f;  // rows past the end already have lse = +inf
+          for (int e = 0; e < 4; e++) {
+            const int i = 4 * i4 + e;
+            const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[i], a.scale_log2, -l4[e]));
+            sacc[i] = p;
+            pacc[i] = p * (pacc[i] - d4[e]);
           }
-          sacc[i] = p;
-          pacc[i] = p * (pacc[i] - d4[e]);
+        }
+      } else {
+        // key position relative to the aligned diagonal of row iw0: rel(r) = rel0 - r
+        const int rel0 = jc - iw0 - shift;
+        const int rel_hi = (a.wr < 0) ? (1 << 30) : a.wr;
+        const int rel_lo = (a.wl < 0 || jc < a.n_sink) ? -(1 << 30) : -a.wl;
+        const int rows_ok = (jc < len_k) ? len_q - iw0 : 0;  // rows r < rows_ok are real
+#pragma unroll
+        for (int i4 = 0; i4 < 4; i4++) {
+          const int rbase = 8 * i4 + 4 * g;
+          const f32x4 l4 = *(const f32x4*)(lse_lds + rbase);
+          const f32x4 d4 = *(const f32x4*)(delta_lds + rbase);
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            const int i = 4 * i4 + e;
+            const int r = rbase + e;
+            const int rel = rel0 - r;
+            const bool ok = (r < rows_ok) & (rel <= rel_hi) & (rel >= rel_lo);
+            float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[i], a.scale_log2, -l4[e]));
+            p = ok ? p : 0.f;
+            sacc[i] = p;
+            pacc[i] = ok ? p * (pacc[i] - d4[e]) : 0.f;
+          }
         }
       }
 
@@ -252,55 +278,55 @@ __global__ __launch_bounds__(512) void attn_bwd_dkdv_kernel(const AttnArgs a) {
         }
         const V8 pb = M::pack(pv);
         const V8 dsb = M::pack(dsv);
-        const int rowoff = (wq * 32 + ks * 16) * C::ROWB;
 #pragma unroll
         for (int d = 0; d < C::DBLK; d++) {
-          const int off0 = (t_row0 ^ (d << 6)) + rowoff;
-          const int off1 = (t_row1 ^ (d << 6)) + rowoff;
+          const int off0 = (t_row0 ^ (d << 6)) + ks * 16 * C::ROWB;
+          const int off1 = (t_row1 ^ (d << 6)) + ks * 16 * C::ROWB;
           dv_acc[d] = M::mfma32(tr_pair<V8>(do_lds + off0, do_lds + off1), pb, dv_acc[d]);
           dk_acc[d] = M::mfma32(tr_pair<V8>(q_lds + off0, q_lds + off1), dsb, dk_acc[d]);
         }
       }
     }
-
-    if (it + 1 < n_iter) store_stats(buf ^ 1);
     __syncthreads();
+  };
+
+  for (int it = 0; it < n_iter; it += 2) {
+    step(it, q_s0, do_s0, st_s0, q_s1, do_s1, st_s1);
+    if (it + 1 < n_iter) step(it + 1, q_s1, do_s1, st_s1, q_s0, do_s0, st_s0);
   }
 
   // ---- add the two query halves (through LDS), then write dK, dV --------------------
-  // (C layout: lane = key, regs = d)
-  float* red = (float*)(smem + wk * C::RED_PER_WK);
-  if (wq == 1) {
+  // (C layout: lane = key, regs = d).  Key groups 0-1 stage in the K tile, 2-3 in the V tile.
+  float* red = (float*)((wk < 2 ? k_s : v_s) + (wk & 1) * C::RED_PER_WK);
 #pragma unroll
-    for (int d = 0; d < C::DBLK; d++)
+  for (int m = 0; m < 2; m++) {  // m = 0: dK, m = 1: dV
+    f32x16* acc = m == 0 ? dk_acc : dv_acc;
+    if (wq == 1) {
 #pragma unroll
-      for (int i4 = 0; i4 < 4; i4++) {
-        const f32x4 kk = {dk_acc[d][4 * i4], dk_acc[d][4 * i4 + 1], dk_acc[d][4 * i4 + 2],
-                          dk_acc[d][4 * i4 + 3]};
-        const f32x4 vv = {dv_acc[d][4 * i4], dv_acc[d][4 * i4 + 1], dv_acc[d][4 * i4 + 2],
-                          dv_acc[d][4 * i4 + 3]};
-        *(f32x4*)(red + ((d * 4 + i4) * 64 + lane) * 4) = kk;
-        *(f32x4*)(red + ((C::DBLK * 4 + d * 4 + i4) * 64 + lane) * 4) = vv;
-      }
-  }
-  __syncthreads();
-  if (wq == 0 && jc < len_k) {
+      for (int d = 0; d < C::DBLK; d++)
 #pragma unroll
-    for (int d = 0; d < C::DBLK; d++)
+        for (int i4 = 0; i4 < 4; i4++) {
+          const f32x4 x = {acc[d][4 * i4], acc[d][4 * i4 + 1], acc[d][4 * i4 + 2],
+                           acc[d][4 * i4 + 3]};
+          *(f32x4*)(red + ((d * 4 + i4) * 64 + lane) * 4) = x;
+        }
+    }
+    __syncthreads();
+    if (wq == 0 && jc < len_k) {
+      const float sc = m == 0 ? a.scale : 1.f;
+      T* dst = (m == 0 ? dk_ptr + (int64_t)jc * a.dk_st[1] : dv_ptr + (int64_t)jc * a.dv_st[1]);
 #pragma unroll
-      for (int i4 = 0; i4 < 4; i4++) {
-        const f32x4 kk = *(const f32x4*)(red + ((d * 4 + i4) * 64 + lane) * 4);
-        const f32x4 vv = *(const f32x4*)(red + ((C::DBLK * 4 + d * 4 + i4) * 64 + lane) * 4);
-        const int col = d * 32 + 8 * i4 + 4 * g;
-        const auto k4 = M::pack4((dk_acc[d][4 * i4] + kk[0]) * a.scale,
-                                 (dk_acc[d][4 * i4 + 1] + kk[1]) * a.scale,
-                                 (dk_acc[d][4 * i4 + 2] + kk[2]) * a.scale,
-                                 (dk_acc[d][4 * i4 + 3] + kk[3]) * a.scale);
-        const auto v4 = M::pack4(dv_acc[d][4 * i4] + vv[0], dv_acc[d][4 * i4 + 1] + vv[1],
-                                 dv_acc[d][4 * i4 + 2] + vv[2], dv_acc[d][4 * i4 + 3] + vv[3]);
-        *(typename M::V4*)(dk_ptr + (int64_t)jc * a.dk_st[1] + col) = k4;
-        *(typename M::V4*)(dv_ptr + (int64_t)jc * a.dv_st[1] + col) = v4;
-      }
+      for (int d = 0; d < C::DBLK; d++)
+#pragma unroll
+        for (int i4 = 0; i4 < 4; i4++) {
+          const f32x4 x = *(const f32x4*)(red + ((d * 4 + i4) * 64 + lane) * 4);
+          const auto h4 = M::pack4((acc[d][4 * i4] + x[0]) * sc, (acc[d][4 * i4 + 1] + x[1]) * sc,
+                                   (acc[d][4 * i4 + 2] + x[2]) * sc,
+                                   (acc[d][4 * i4 + 3] + x[3]) * sc);
+          *(typename M::V4*)(dst + d * 32 + 8 * i4 + 4 * g) = h4;
+        }
+    }
+    __syncthreads();
   }
 }
 
@@ -309,28 +335,26 @@ __global__ __launch_bounds__(512) void attn_bwd_dkdv_kernel(const AttnArgs a) {
 // ============================================================================
 template <int D>
 struct DqCfg {
-  static constexpr int BM = 128;  // query rows per block
-  static constexpr int BN = 64;   // keys per step
-  static constexpr int THREADS = 256;
+  static constexpr int BN = 64;  // keys per step
+  static constexpr int THREADS = 512;
   static constexpr int KSTEPS = D / 16;
   static constexpr int DBLK = D / 32;
   static constexpr int CPR = D / 8;
   static constexpr int ROWB = D * 2;
-  static constexpr int CH = BN * CPR / THREADS;
   static constexpr int TILE = BN * ROWB;
-  static constexpr int OFF_K = 0;         // 2 buffers
-  static constexpr int OFF_V = 2 * TILE;  // 2 buffers
-  static constexpr int SMEM = 4 * TILE;
   static constexpr int O_STRIDE = D * 2 + 16;
-  static_assert(SMEM >= 4 * 32 * O_STRIDE, "epilogue staging must fit");
+  static_assert(TILE >= 32 * O_STRIDE, "one wave's epilogue staging fits one tile buffer");
 };
 
 template <typename T, int D>
-__global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
+__global__ __launch_bounds__(512) void attn_bwd_dq_kernel(const AttnArgs a) {
   using C = DqCfg<D>;
   using M = Mma<T>;
   using V8 = typename M::V8;
-  extern __shared__ __attribute__((aligned(16))) char smem[];
+  __shared__ __attribute__((aligned(1024))) char k_s0[C::TILE];
+  __shared__ __attribute__((aligned(1024))) char k_s1[C::TILE];
+  __shared__ __attribute__((aligned(1024))) char v_s0[C::TILE];
+  __shared__ __attribute__((aligned(1024))) char v_s1[C::TILE];
 
   const int wid = logical_block_id(a.n_work);
   if (wid < 0) return;
@@ -342,16 +366,21 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
   const int i16 = lane & 15;
   const int u = lane >> 4;
 
-  const int hg = wid % a.group;
-  int rest = wid / a.group;
+  // pair mode: waves 0-3 and 4-7 take the same 128 rows of two neighbouring q heads;
+  // row mode: the 8 waves take 256 consecutive rows of one q head
+  const bool pair = (a.group & 1) == 0;
+  const int units = pair ? a.group >> 1 : a.group;
+  const int bm = pair ? 128 : 256;
+  const int hu = wid % units;
+  int rest = wid / units;
   const int slot = rest % a.n_tile;
   rest /= a.n_tile;
   const int hk = rest % a.heads_kv;
-  const int hq = hk * a.group + hg;
+  const int hq = hk * a.group + (pair ? 2 * hu + (wave >> 2) : hu);
   SeqInfo s;
   int qt;
   if (a.cu_q) {
-    if (!locate_packed(a, slot, C::BM, false, s, qt)) return;
+    if (!locate_packed(a, slot, bm, false, s, qt)) return;
   } else {
     s.batch_idx = rest / a.heads_kv;
     s.q_row0 = s.k_row0 = 0;
@@ -361,7 +390,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
   }
   const int b = s.batch_idx;
   const int len_q = s.len_q, len_k = s.len_k;
-  const int i0 = qt * C::BM;
+  const int i0 = qt * bm;
   if (i0 >= len_q) return;
 
   const T* q_ptr = (const T*)a.q + b * a.q_st[0] + s.q_row0 * a.q_st[1] + hq * a.q_st[2];
@@ -372,7 +401,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
   const int64_t ws_row0 = a.cu_q ? s.q_row0 : (int64_t)b * a.seqlen_q;
 
   // ---- key tiles this block visits (same rule as the forward kernel) -----------
-  const int i_last = min(i0 + C::BM, len_q) - 1;
+  const int i_last = min(i0 + bm, len_q) - 1;
   const int lo_blk = row_bounds(a, i0, len_q, len_k).lo;
   const int hi_blk = row_bounds(a, i_last, len_q, len_k).hi;
   const bool band = hi_blk >= lo_blk;
@@ -383,7 +412,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
   const int n_tiles = n_sink_t + n_band;
   auto tile_of = [&](int it) { return it < n_sink_t ? it : t_lo + (it - n_sink_t); };
 
-  const int r0 = i0 + wave * 32;
+  const int r0 = i0 + (pair ? wave & 3 : wave) * 32;
   const int iq = r0 + l32;
   const RowBounds rb = row_bounds(a, iq, len_q, len_k);
   const bool wave_valid = r0 < len_q;
@@ -400,8 +429,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
       qf[ks] = *(const V8*)(q_ptr + (int64_t)iq * a.q_st[1] + ks * 16 + g * 8);
       dof[ks] = *(const V8*)(do_ptr + (int64_t)iq * a.do_st[1] + ks * 16 + g * 8);
     }
-    const float l = a.lse[b * a.lse_st[0] + hq * a.lse_st[1] + (s.q_row0 + iq) * a.lse_st[2]];
-    lse2 = (l == -__builtin_inff()) ? __builtin_inff() : l * kLog2e;
+    lse2 = a.lse2[(int64_t)hq * a.rows_q + ws_row0 + iq];
     delta = a.delta[(int64_t)hq * a.rows_q + ws_row0 + iq];
   } else {
 #pragma unroll
@@ -417,50 +445,32 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
 #pragma unroll
     for (int i = 0; i < 16; i++) dq_acc[d][i] = 0.f;
 
-  u32x4 kreg[C::CH], vreg[C::CH];
-  auto load_tile = [&](int tile) {
-    const int j0 = tile * C::BN;
-#pragma unroll
-    for (int n = 0; n < C::CH; n++) {
-      const int c = tid + n * C::THREADS;
-      const int row = c / C::CPR, col = (c % C::CPR) * 8;
-      if (j0 + row < len_k) {
-        kreg[n] = *(const u32x4*)(k_ptr + (int64_t)(j0 + row) * a.k_st[1] + col);
-        vreg[n] = *(const u32x4*)(v_ptr + (int64_t)(j0 + row) * a.v_st[1] + col);
-      } else {
-        kreg[n] = u32x4{0, 0, 0, 0};
-        vreg[n] = u32x4{0, 0, 0, 0};
-      }
-    }
-  };
-  auto store_tile = [&](int buf) {
-#pragma unroll
-    for (int n = 0; n < C::CH; n++) {
-      const int c = tid + n * C::THREADS;
-      const int row = c / C::CPR, ch = c % C::CPR;
-      const int off = row * C::ROWB + swz<C::CPR>(row, ch) * 16;
-      *(u32x4*)(smem + C::OFF_K + buf * C::TILE + off) = kreg[n];
-      *(u32x4*)(smem + C::OFF_V + buf * C::TILE + off) = vreg[n];
-    }
+  // lane-constant LDS offsets (see the forward kernel)
+  const int a_row = l32 * C::ROWB + ((g ^ swz_f<C::CPR>(l32)) << 4);
+  const int rl = 4 * g + (i16 >> 2);
+  const int lp = 2 * (u & 1) + ((i16 & 3) >> 1);
+  const int t_row0 = rl * C::ROWB + ((lp ^ swz_f<C::CPR>(rl)) << 4) + (i16 & 1) * 8;
+  const int t_row1 = (rl + 8) * C::ROWB + ((lp ^ swz_f<C::CPR>(rl + 8)) << 4) + (i16 & 1) * 8;
+
+  const __amdgpu_buffer_rsrc_t k_rsrc = make_rows_rsrc(k_ptr, len_k, a.k_st[1] * 2, C::ROWB);
+  const __amdgpu_buffer_rsrc_t v_rsrc = make_rows_rsrc(v_ptr, len_k, a.v_st[1] * 2, C::ROWB);
+  TileDma<D, C::BN, C::THREADS> k_dma, v_dma;
+  k_dma.init(a.k_st[1], tid);
+  v_dma.init(a.v_st[1], tid);
+  const int k_tile_bytes = (int)(C::BN * a.k_st[1] * 2), v_tile_bytes = (int)(C::BN * a.v_st[1] * 2);
+  auto load_tile = [&](int it, char* kd, char* vd) __attribute__((always_inline)) {
+    k_dma.load(k_rsrc, tile_of(it) * k_tile_bytes, kd);
+    v_dma.load(v_rsrc, tile_of(it) * v_tile_bytes, vd);
   };
 
-  if (n_tiles > 0) {
-    load_tile(tile_of(0));
-    store_tile(0);
-  }
-  __syncthreads();
-
-  for (int it = 0; it < n_tiles; it++) {
-    const int buf = it & 1;
+  auto step = [&](int it, const char* kc, const char* vc, char* kn,
+                  char* vn) __attribute__((always_inline)) {
     const int j0 = tile_of(it) * C::BN;
     const int j1 = j0 + C::BN - 1;
-    if (it + 1 < n_tiles) load_tile(tile_of(it + 1));
-
+    if (it + 1 < n_tiles) load_tile(it + 1, kn, vn);
     const bool needed =
         wave_valid && j0 <= wb_last.hi && (j1 >= wb_first.lo || j0 < a.n_sink);
     if (needed) {
-      const char* k_lds = smem + C::OFF_K + buf * C::TILE;
-      const char* v_lds = smem + C::OFF_V + buf * C::TILE;
       // S^T = K Q^T and dP^T = V dO^T (rows = keys, lane = query column)
       f32x16 sacc[2], pacc[2];
 #pragma unroll
@@ -472,75 +482,96 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
         }
 #pragma unroll
       for (int ks = 0; ks < C::KSTEPS; ks++) {
+        const int off = a_row ^ (ks << 5);
 #pragma unroll
         for (int t = 0; t < 2; t++) {
-          const int row = t * 32 + l32;
-          const int off = row * C::ROWB + swz<C::CPR>(row, ks * 2 + g) * 16;
-          sacc[t] = M::mfma32(*(const V8*)(k_lds + off), qf[ks], sacc[t]);
-          pacc[t] = M::mfma32(*(const V8*)(v_lds + off), dof[ks], pacc[t]);
+          sacc[t] = M::mfma32(*(const V8*)(kc + off + t * 32 * C::ROWB), qf[ks], sacc[t]);
+          pacc[t] = M::mfma32(*(const V8*)(vc + off + t * 32 * C::ROWB), dof[ks], pacc[t]);
         }
       }
       const bool full = wave_rows_full && j1 <= wb_first.hi &&
                         (j0 >= wb_last.lo || j1 < a.n_sink);
+      if (full) {
 #pragma unroll
-      for (int t = 0; t < 2; t++)
+        for (int t = 0; t < 2; t++)
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-          float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[t][i], a.scale_log2, -lse2));
-          if (!full) {
-            const int j = j0 + t * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
-            const bool ok = j <= rb.hi && (j >= rb.lo || j < a.n_sink);
-            p = ok ? p : 0.f;
+          for (int i = 0; i < 16; i++) {
+            const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[t][i], a.scale_log2, -lse2));
+            pacc[t][i] = p * (pacc[t][i] - delta);
           }
-          pacc[t][i] = p * (pacc[t][i] - delta);
-        }
+      } else {
+        const int hi_rel = rb.hi - j0;
+        const int lo_rel = rb.lo - j0;
+        const int sink_rel = a.n_sink - j0;
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+          for (int i = 0; i < 16; i++) {
+            const int j = t * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
+            const bool ok = (j <= hi_rel) & ((j >= lo_rel) | (j < sink_rel));
+            const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[t][i], a.scale_log2, -lse2));
+            pacc[t][i] = ok ? p * (pacc[t][i] - delta) : 0.f;
+          }
+      }
       // dQ^T[d, query] += K^T dS^T
-      const int rlane = 4 * g + (i16 >> 2);
-      const int half = (i16 & 1) * 8;
 #pragma unroll
       for (int s4 = 0; s4 < 4; s4++) {
         float dsv[8];
 #pragma unroll
         for (int j = 0; j < 8; j++) dsv[j] = pacc[s4 >> 1][8 * (s4 & 1) + j];
         const V8 dsb = M::pack(dsv);
-        const int row = s4 * 16 + rlane;
 #pragma unroll
         for (int d = 0; d < C::DBLK; d++) {
-          const int ch = 4 * d + 2 * (u & 1) + ((i16 & 3) >> 1);
-          const int off0 = row * C::ROWB + swz<C::CPR>(row, ch) * 16 + half;
-          const int off1 = (row + 8) * C::ROWB + swz<C::CPR>(row + 8, ch) * 16 + half;
-          dq_acc[d] = M::mfma32(tr_pair<V8>(k_lds + off0, k_lds + off1), dsb, dq_acc[d]);
+          const int off0 = (t_row0 ^ (d << 6)) + s4 * 16 * C::ROWB;
+          const int off1 = (t_row1 ^ (d << 6)) + s4 * 16 * C::ROWB;
+          dq_acc[d] = M::mfma32(tr_pair<V8>(kc + off0, kc + off1), dsb, dq_acc[d]);
         }
       }
     }
-    if (it + 1 < n_tiles) store_tile(buf ^ 1);
     __syncthreads();
+  };
+
+  if (n_tiles > 0) load_tile(0, k_s0, v_s0);
+  __syncthreads();
+  for (int it = 0; it < n_tiles; it += 2) {
+    step(it, k_s0, v_s0, k_s1, v_s1);
+    if (it + 1 < n_tiles) step(it + 1, k_s1, v_s1, k_s0, v_s0);
   }
 
   // ---- epilogue: dq = scale * acc, transposed through LDS for 16-byte stores ------
-  char* stage = smem + wave * 32 * C::O_STRIDE;
+  char* stage = (wave & 3) == 0 ? k_s0 : (wave & 3) == 1 ? k_s1 : (wave & 3) == 2 ? v_s0 : v_s1;
+  for (int half = 0; half < 2; half++) {
+    if ((wave >> 2) == half) {
 #pragma unroll
-  for (int d = 0; d < C::DBLK; d++)
+      for (int d = 0; d < C::DBLK; d++)
 #pragma unroll
-    for (int i4 = 0; i4 < 4; i4++) {
-      const auto h4 = M::pack4(dq_acc[d][4 * i4] * a.scale, dq_acc[d][4 * i4 + 1] * a.scale,
-                               dq_acc[d][4 * i4 + 2] * a.scale, dq_acc[d][4 * i4 + 3] * a.scale);
-      *(typename M::V4*)(stage + l32 * C::O_STRIDE + (d * 32 + 8 * i4 + 4 * g) * 2) = h4;
+        for (int i4 = 0; i4 < 4; i4++) {
+          const auto h4 =
+              M::pack4(dq_acc[d][4 * i4] * a.scale, dq_acc[d][4 * i4 + 1] * a.scale,
+                       dq_acc[d][4 * i4 + 2] * a.scale, dq_acc[d][4 * i4 + 3] * a.scale);
+          *(typename M::V4*)(stage + l32 * C::O_STRIDE + (d * 32 + 8 * i4 + 4 * g) * 2) = h4;
+        }
     }
-  __syncthreads();
+    __syncthreads();
+    if ((wave >> 2) == half) {
 #pragma unroll
-  for (int n = 0; n < 32 * C::CPR / 64; n++) {
-    const int c = lane + n * 64;
-    const int row = c / C::CPR, col = (c % C::CPR) * 8;
-    if (r0 + row < len_q) {
-      const u32x4 val = *(const u32x4*)(stage + row * C::O_STRIDE + col * 2);
-      *(u32x4*)(dq_ptr + (int64_t)(r0 + row) * a.dq_st[1] + col) = val;
+      for (int n = 0; n < 32 * C::CPR / 64; n++) {
+        const int c = lane + n * 64;
+        const int row = c / C::CPR, col = (c % C::CPR) * 8;
+        if (r0 + row < len_q) {
+          const u32x4 val = *(const u32x4*)(stage + row * C::O_STRIDE + col * 2);
+          *(u32x4*)(dq_ptr + (int64_t)(r0 + row) * a.dq_st[1] + col) = val;
+        }
+      }
     }
+    __syncthreads();
   }
 }
 
 // ============================================================================
-// delta[h][row] = sum_d dO * O.  One 16-lane (D=128) or 8-lane (D=64) group per (row, head).
+// row statistics: delta = sum_d dO * O and lse2 = lse * log2(e) (empty rows: +inf, so
+// that P = exp2(S*c - lse2) is zero).  One 16-lane (D=128) or 8-lane (D=64) group per
+// (row, head).
 // ============================================================================
 template <typename T, int D>
 __global__ __launch_bounds__(256) void attn_bwd_prep_kernel(const AttnArgs a) {
@@ -550,14 +581,16 @@ __global__ __launch_bounds__(256) void attn_bwd_prep_kernel(const AttnArgs a) {
   if (unit >= a.rows_q * a.heads_q) return;
   const int h = (int)(unit % a.heads_q);
   const int64_t row = unit / a.heads_q;
-  int64_t o_off, do_off;
+  int64_t o_off, do_off, l_off;
   if (a.cu_q) {
     o_off = row * a.o_st[1];
     do_off = row * a.do_st[1];
+    l_off = row * a.lse_st[2];
   } else {
     const int64_t bb = row / a.seqlen_q, i = row % a.seqlen_q;
     o_off = bb * a.o_st[0] + i * a.o_st[1];
     do_off = bb * a.do_st[0] + i * a.do_st[1];
+    l_off = bb * a.lse_st[0] + i * a.lse_st[2];
   }
   using V8 = typename Mma<T>::V8;
   const V8 o8 = *(const V8*)((const T*)a.out + o_off + h * a.o_st[2] + c);
@@ -567,19 +600,24 @@ __global__ __launch_bounds__(256) void attn_bwd_prep_kernel(const AttnArgs a) {
   for (int j = 0; j < 8; j++) acc += (float)o8[j] * (float)d8[j];
 #pragma unroll
   for (int m = LPR / 2; m >= 1; m >>= 1) acc += __shfl_xor(acc, m, 64);
-  if (c == 0) a.delta[(int64_t)h * a.rows_q + row] = acc;
+  if (c == 0) {
+    a.delta[(int64_t)h * a.rows_q + row] = acc;
+    const float l = a.lse[l_off + h * a.lse_st[1]];
+    a.lse2[(int64_t)h * a.rows_q + row] = (l == -__builtin_inff()) ? __builtin_inff() : l * kLog2e;
+  }
 }
 
-template <typename Kern>
-int set_smem(Kern kern, int bytes, bool& configured, const char* what) {
-  if (!configured) {  // benign race: the attribute call is idempotent
-    hipError_t e =
-        hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-    if (e != hipSuccess) return fail(RSWA_ERR_LAUNCH, "%s: set smem: %s", what, hipGetErrorString(e));
-    configured = true;
-  }
-  return RSWA_OK;
-}
+// Explicit instantiations: with implicit instantiation alone this hipcc emits the host
+// launch stubs of only some of the variants.
+#define RSWA_INSTANTIATE(T, D)                                              \
+  template __global__ void attn_bwd_dkdv_kernel<T, D>(const AttnArgs);      \
+  template __global__ void attn_bwd_dq_kernel<T, D>(const AttnArgs);        \
+  template __global__ void attn_bwd_prep_kernel<T, D>(const AttnArgs);
+RSWA_INSTANTIATE(__bf16, 128)
+RSWA_INSTANTIATE(__bf16, 64)
+RSWA_INSTANTIATE(_Float16, 128)
+RSWA_INSTANTIATE(_Float16, 64)
+#undef RSWA_INSTANTIATE
 
 template <typename T, int D>
 int launch_bwd(AttnArgs& a, hipStream_t stream, int phases) {
@@ -600,31 +638,28 @@ int launch_bwd(AttnArgs& a, hipStream_t stream, int phases) {
       a.n_work = a.n_tile * a.heads_kv * a.batch;
     }
     if (a.n_work > 0) {
-      auto kern = attn_bwd_dkdv_kernel<T, D>;
-      static bool configured = false;
-      int rc = set_smem(kern, C::SMEM, configured, "attn_bwd dkdv");
-      if (rc != RSWA_OK) return rc;
-      hipLaunchKernelGGL(kern, dim3(padded_grid(a.n_work)), dim3(C::THREADS), C::SMEM, stream, a);
-      rc = check_launch("attn_bwd dkdv");
+      hipLaunchKernelGGL((attn_bwd_dkdv_kernel<T, D>), dim3(padded_grid(a.n_work)),
+                         dim3(C::THREADS), 0, stream, a);
+      int rc = check_launch("attn_bwd dkdv");
       if (rc != RSWA_OK) return rc;
     }
   }
   if (phases & RSWA_BWD_DQ) {
     using C = DqCfg<D>;
+    const bool pair = (a.group & 1) == 0;
+    const int bm = pair ? 128 : 256;
+    const int units_q = (pair ? a.group / 2 : a.group) * a.heads_kv;  // blocks per q tile
     if (a.cu_q) {
-      a.n_tile = (int)(ceil_div(a.rows_q, C::BM) + a.batch);
-      a.n_work = a.n_tile * a.heads_q;
+      a.n_tile = (int)(ceil_div(a.rows_q, bm) + a.batch);
+      a.n_work = a.n_tile * units_q;
     } else {
-      a.n_tile = (int)ceil_div(a.seqlen_q, C::BM);
-      a.n_work = a.n_tile * a.heads_q * a.batch;
+      a.n_tile = (int)ceil_div(a.seqlen_q, bm);
+      a.n_work = a.n_tile * units_q * a.batch;
     }
     if (a.n_work > 0) {
-      auto kern = attn_bwd_dq_kernel<T, D>;
-      static bool configured = false;
-      int rc = set_smem(kern, C::SMEM, configured, "attn_bwd dq");
-      if (rc != RSWA_OK) return rc;
-      hipLaunchKernelGGL(kern, dim3(padded_grid(a.n_work)), dim3(C::THREADS), C::SMEM, stream, a);
-      rc = check_launch("attn_bwd dq");
+      hipLaunchKernelGGL((attn_bwd_dq_kernel<T, D>), dim3(padded_grid(a.n_work)),
+                         dim3(C::THREADS), 0, stream, a);
+      int rc = check_launch("attn_bwd dq");
       if (rc != RSWA_OK) return rc;
     }
   }

@@ -29,7 +29,8 @@ struct AttnArgs {
   void* dq;
   void* dk;
   void* dv;
-  float* delta;   // fp32 [heads_q, rows_q] packed, inside the workspace
+  float* delta;   // fp32 [heads_q, rows_q] packed: sum_d dO * O          (workspace)
+  float* lse2;    // fp32 [heads_q, rows_q] packed: lse * log2(e), -inf -> +inf (workspace)
   const int32_t* cu_q;
   const int32_t* cu_k;
   int64_t q_st[3], k_st[3], v_st[3], o_st[3], do_st[3], dq_st[3], dk_st[3], dv_st[3], lse_st[3];
