@@ -176,32 +176,6 @@ __device__ __forceinline__ V8 tr_pair(const char* p0, const char* p1) {
 }
 
 typedef __attribute__((address_space(3))) void lds_void_t;
-typedef __attribute__((address_space(1))) const void glob_void_t;
-
-// Cooperative copy of a [ROWS x D] tile (row-major in global memory, `stride` elements
-// between rows) into a swizzled LDS tile with direct global->LDS loads
-// (global_load_lds_dwordx4: lane L of a wave lands at wave_base + 16 L): no staging
-// registers, no LDS store instructions.  Rows >= valid_rows repeat row valid_rows - 1
-// (finite data the mask never lets through); valid_rows must be >= 1.
-template <typename T, int D, int ROWS, int THREADS>
-__device__ __forceinline__ void g2lds_tile(const T* src, int64_t stride, int valid_rows,
-                                           char* lds_tile, int tid) {
-  constexpr int CPR = D / 8;
-  constexpr int RPI = 64 / CPR;  // rows per wave instruction
-  constexpr int NW = THREADS / 64;
-  constexpr int N = ROWS * CPR / THREADS;
-  static_assert(N * THREADS == ROWS * CPR, "tile must divide evenly");
-  const int lane = tid & 63, wave = tid >> 6;
-#pragma unroll
-  for (int n = 0; n < N; n++) {
-    const int slot = n * NW + wave;
-    const int row = slot * RPI + lane / CPR;
-    const int lc = (lane % CPR) ^ swz_f<CPR>(row);
-    const int rr = min(row, valid_rows - 1);
-    __builtin_amdgcn_global_load_lds((glob_void_t*)(src + (int64_t)rr * stride + lc * 8),
-                                     (lds_void_t*)(lds_tile + slot * 1024), 16, 0, 0);
-  }
-}
 
 // Buffer resource over the rows of one (sequence, head) slice: `rows` rows of `row_bytes`
 // useful bytes, `stride_bytes` apart.  Loads past the last row return zero, in registers
@@ -244,6 +218,16 @@ struct TileDma {
     }
   }
 };
+
+// Block barrier that waits for this wave's LDS traffic only: loads still in flight from
+// global memory into LDS (vmcnt) are NOT drained, unlike __syncthreads().  A wave that
+// issued such loads calls wait_dma() before the barrier that publishes them.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+__device__ __forceinline__ void wait_dma() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 // max / sum across the two half-waves (lane l <-> lane l ^ 32).
 __device__ __forceinline__ float halfwave_max(float x) {

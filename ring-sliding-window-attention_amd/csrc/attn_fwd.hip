@@ -200,12 +200,17 @@ __global__ __launch_bounds__(512) void attn_fwd_kernel(const AttnArgs a) {
 #pragma unroll
       for (int i = 0; i < 16; i++) mx = fmaxf(mx, sacc[t][i]);
     mx = halfwave_max(mx);
+    // The reference point of the exponentials moves only when the maximum has grown by
+    // more than 2^8: until then P <= 256, exact in fp32 sums and harmless in 16 bits, and
+    // the rescale of the running output is skipped for almost every tile.
     const float m_new = fmaxf(m_run, mx);
-    const float m_use = (m_new == -__builtin_inff()) ? 0.f : m_new;
+    const bool bump = (m_new - m_run) * a.scale_log2 > 8.f;  // true from -inf, false for NaN
+    const float m_keep = bump ? m_new : m_run;
+    const float m_use = (m_keep == -__builtin_inff()) ? 0.f : m_keep;
     const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * a.scale_log2);
     const float mc = m_use * a.scale_log2;
-    m_run = m_new;
-    float psum = 0.f;
+    m_run = m_keep;
+    float psum[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s4 = 0; s4 < 4; s4++) {
       float pv[8];
@@ -213,21 +218,27 @@ __global__ __launch_bounds__(512) void attn_fwd_kernel(const AttnArgs a) {
       for (int j = 0; j < 8; j++) {
         pv[j] = __builtin_amdgcn_exp2f(
             __builtin_fmaf(sacc[s4 >> 1][8 * (s4 & 1) + j], a.scale_log2, -mc));
-        psum += pv[j];
+        psum[j & 3] += pv[j];
       }
       pb[s4] = M::pack(pv);
+      // keep the vector work in the vector phase: the packed P is opaque from here on
+      asm volatile("" : "+v"(pb[s4]));
     }
-    l_run = l_run * alpha + psum;
+    float psum_all = (psum[0] + psum[1]) + (psum[2] + psum[3]);
+    asm volatile("" : "+v"(psum_all));
+    l_run = l_run * alpha + psum_all;
     return alpha;
   };
-  // O^T[d, query] = alpha * O^T + V^T P^T
-  auto pv_acc = [&](const char* vc, const V8(&pb)[4], float alpha) __attribute__((always_inline)) {
+  // O^T[d, query] = alpha * O^T + V^T P^T, in two parts
+  auto rescale = [&](float alpha) __attribute__((always_inline)) {
     if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {
 #pragma unroll
       for (int d = 0; d < C::DBLK; d++)
 #pragma unroll
         for (int i = 0; i < 16; i++) o_acc[d][i] *= alpha;
     }
+  };
+  auto pv_acc = [&](const char* vc, const V8(&pb)[4]) __attribute__((always_inline)) {
 #pragma unroll
     for (int s4 = 0; s4 < 4; s4++) {
 #pragma unroll
@@ -239,28 +250,48 @@ __global__ __launch_bounds__(512) void attn_fwd_kernel(const AttnArgs a) {
     }
   };
 
-  // ---- pipelined tile loop ----------------------------------------------------------
-  // entering step(t): S(t) is in s_cur; K(t+1) and V(t) are in LDS (kn, vc); the buffer kc
-  // that held K(t) is free.  The step starts the loads of K(t+2) -> kc and V(t+1) -> vn,
-  // computes S(t+1) under the softmax of tile t, accumulates P(t) V(t), and syncs.
-  f32x16 s_cur[2], s_nxt[2];
-  auto step = [&](int it, char* kc, const char* kn, const char* vc,
-                  char* vn) __attribute__((always_inline)) {
-    if (it + 2 < n_tiles) load_k(it + 2, kc);
+  // ---- ping-pong tile loop ------------------------------------------------------------
+  // A wave alternates a vector phase (mask + softmax of tile t, rescale of O) and a matrix
+  // phase (O += P(t) V(t), S(t+1) = K(t+1) Q^T), with a block barrier after each.  Waves 4-7
+  // run one phase behind waves 0-3, so on every SIMD one wave is in its matrix phase
+  // while the other is in its vector phase and both pipes stay busy.
+  // Tile loads: the wave group that is in the phase slot after both groups have finished
+  // reading K(t), V(t-1) issues K(t+2) and V(t+1) into those buffers and waits for them
+  // before the barrier that precedes their first use, one full slot later.
+  const bool late = __builtin_amdgcn_readfirstlane(wave >> 2) != 0;
+  f32x16 s_cur[2];
+  auto prefetch = [&](int it, char* kfree, char* vn) __attribute__((always_inline)) {
+    if (it + 2 < n_tiles) load_k(it + 2, kfree);
     if (it + 1 < n_tiles) load_v(it + 1, vn);
+  };
+  auto iter = [&](int it, const char* kn, char* kfree, const char* vc,
+                  char* vn) __attribute__((always_inline)) {
+    if (late) prefetch(it, kfree, vn);
     mask(it, s_cur);
     V8 pb[4];
-    float alpha;
-    if (it + 1 < n_tiles) {
-      qk(kn, s_nxt);
-      alpha = softmax(s_cur, pb);
-    } else {
-      alpha = softmax(s_cur, pb);
-    }
-    pv_acc(vc, pb, alpha);
+    const float alpha = softmax(s_cur, pb);
+    rescale(alpha);
+    if (!late) wait_dma();
+    lds_barrier();
+    if (!late) prefetch(it, kfree, vn);
+    // matrix phase as ONE basic block (after the last tile S(t+1) is computed from stale
+    // LDS contents and never used), LDS reads scheduled four fragments ahead of their MFMA
+    pv_acc(vc, pb);
+    qk(kn, s_cur);
+    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
 #pragma unroll
-    for (int t = 0; t < 2; t++) s_cur[t] = s_nxt[t];
-    __syncthreads();
+    for (int i = 0; i < 12; i++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+    if (late) wait_dma();
+    lds_barrier();
   };
 
   if (n_tiles > 0) {
@@ -269,12 +300,15 @@ __global__ __launch_bounds__(512) void attn_fwd_kernel(const AttnArgs a) {
   }
   if (n_tiles > 1) load_k(1, k_s1);
   __syncthreads();
+  if (late) lds_barrier();
   if (n_tiles > 0) qk(k_s0, s_cur);
-  __syncthreads();  // every wave has read K(0) before step(0) overwrites its buffer
+  lds_barrier();
   for (int it = 0; it < n_tiles; it += 2) {
-    step(it, k_s0, k_s1, v_s0, v_s1);
-    if (it + 1 < n_tiles) step(it + 1, k_s1, k_s0, v_s1, v_s0);
+    iter(it, k_s1, k_s0, v_s0, v_s1);
+    if (it + 1 < n_tiles) iter(it + 1, k_s0, k_s1, v_s1, v_s0);
   }
+  if (!late) lds_barrier();
+  __syncthreads();
 
   // ---- epilogue --------------------------------------------------------------
   const float l_tot = halfwave_sum(l_run);
