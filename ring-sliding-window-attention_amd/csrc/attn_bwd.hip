@@ -73,7 +73,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   if (wid < 0) return;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wk = wave & 3;   // key group: columns 32 wk .. 32 wk + 31 of the block's 128 keys
   const int wq = wave >> 2;  // query half: rows 32 wq .. 32 wq + 31 of each 64-row tile
   const int l32 = lane & 31;
@@ -149,29 +149,47 @@ __global__ __launch_bounds__(512) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   do_dma.init(a.do_st[1], tid);
   const T* q_base = (const T*)a.q + b * a.q_st[0] + s.q_row0 * a.q_st[1];
   const T* do_base = (const T*)a.dout + b * a.do_st[0] + s.q_row0 * a.do_st[1];
+  const int q_row_bytes = (int)(a.q_st[1] * 2), do_row_bytes = (int)(a.do_st[1] * 2);
   // statistics: one resource over both workspace arrays (lse2 then delta); rows past the
   // sequence end read a neighbour's finite values, which the row mask / zero Q, dO rows void
   const int64_t stat_elems = a.delta - a.lse2;  // elements between the two arrays
   const __amdgpu_buffer_rsrc_t st_rsrc = __builtin_amdgcn_make_buffer_rsrc(
       (void*)a.lse2, 0, (int)((stat_elems + a.heads_q * a.rows_q) * 4), 0x00020000);
 
-  auto iter_coords = [&](int it, int& hq, int& i0) __attribute__((always_inline)) {
-    hq = hk * a.group + it / n_qt;
-    i0 = (qt_lo + it % n_qt) * C::BM;
+  // Cursor over the (q head of the group, query tile) pairs, advanced incrementally so
+  // that a step costs a handful of scalar instructions: the tile's first row, the head's
+  // Q / dO base pointers and the offset of its statistics.
+  struct Cursor {
+    int qt, i0;
+    const T *q_head, *do_head;
+    int64_t stat_row;  // index of row 0 of this head in the statistics arrays
   };
-  auto load_iter = [&](int it, char* qd, char* dod, float* std_) __attribute__((always_inline)) {
-    int hq, i0;
-    iter_coords(it, hq, i0);
-    const __amdgpu_buffer_rsrc_t q_rsrc =
-        make_rows_rsrc(q_base + hq * a.q_st[2], len_q, a.q_st[1] * 2, C::ROWB);
+  const int i_first = qt_lo * C::BM;
+  Cursor nxt;  // the tile that load_next() fetches
+  nxt.qt = 0;
+  nxt.i0 = i_first;
+  nxt.q_head = q_base + (int64_t)hk * a.group * a.q_st[2];
+  nxt.do_head = do_base + (int64_t)hk * a.group * a.do_st[2];
+  nxt.stat_row = (int64_t)hk * a.group * a.rows_q + ws_row0;
+  auto load_next = [&](char* qd, char* dod, float* std_) __attribute__((always_inline)) {
+    const __amdgpu_buffer_rsrc_t q_rsrc = make_rows_rsrc(nxt.q_head, len_q, a.q_st[1] * 2, C::ROWB);
     const __amdgpu_buffer_rsrc_t do_rsrc =
-        make_rows_rsrc(do_base + hq * a.do_st[2], len_q, a.do_st[1] * 2, C::ROWB);
-    q_dma.load(q_rsrc, (int)(i0 * a.q_st[1] * 2), qd);
-    do_dma.load(do_rsrc, (int)(i0 * a.do_st[1] * 2), dod);
+        make_rows_rsrc(nxt.do_head, len_q, a.do_st[1] * 2, C::ROWB);
+    q_dma.load(q_rsrc, nxt.i0 * q_row_bytes, qd);
+    do_dma.load(do_rsrc, nxt.i0 * do_row_bytes, dod);
     if (wave < 2) {  // wave 0: lse2 tile, wave 1: delta tile (64 floats each)
-      const int soff = (int)(((int64_t)hq * a.rows_q + ws_row0 + i0 + wave * stat_elems) * 4);
+      const int soff = (int)((nxt.stat_row + nxt.i0 + wave * stat_elems) * 4);
       __builtin_amdgcn_raw_ptr_buffer_load_lds(st_rsrc, (lds_void_t*)(std_ + wave * C::BM), 4,
                                                lane * 4, soff, 0, 0);
+    }
+    nxt.qt++;
+    nxt.i0 += C::BM;
+    if (nxt.qt == n_qt) {
+      nxt.qt = 0;
+      nxt.i0 = i_first;
+      nxt.q_head += a.q_st[2];
+      nxt.do_head += a.do_st[2];
+      nxt.stat_row += a.rows_q;
     }
   };
 
@@ -180,19 +198,20 @@ __global__ __launch_bounds__(512) void attn_bwd_dkdv_kernel(const AttnArgs a) {
     const __amdgpu_buffer_rsrc_t v_rsrc = make_rows_rsrc(v_ptr, len_k, a.v_st[1] * 2, C::ROWB);
     k_dma.load(k_rsrc, (int)(j0 * a.k_st[1] * 2), k_s);
     v_dma.load(v_rsrc, (int)(j0 * a.v_st[1] * 2), v_s);
-    load_iter(0, q_s0, do_s0, st_s0);
+    load_next(q_s0, do_s0, st_s0);
   }
   __syncthreads();
 
   const char* k_lds = k_s + wk * 32 * C::ROWB;
   const char* v_lds = v_s + wk * 32 * C::ROWB;
 
+  int cur_i0 = i_first;  // first row of the tile being computed
   // one query tile: prefetch the next one into (qn, don, stn), compute on (qc, doc, stc)
   auto step = [&](int it, const char* qc, const char* doc, const float* stc, char* qn, char* don,
                   float* stn) __attribute__((always_inline)) {
-    int hq, i0;
-    iter_coords(it, hq, i0);
-    if (it + 1 < n_iter) load_iter(it + 1, qn, don, stn);
+    const int i0 = cur_i0;
+    cur_i0 = nxt.i0;  // the tile fetched now is the next step's
+    if (it + 1 < n_iter) load_next(qn, don, stn);
     const char* q_lds = qc + wq * 32 * C::ROWB;
     const char* do_lds = doc + wq * 32 * C::ROWB;
     const float* lse_lds = stc + wq * 32;
@@ -223,6 +242,14 @@ __global__ __launch_bounds__(512) void attn_bwd_dkdv_kernel(const AttnArgs a) {
         sacc = M::mfma32(qa, kb, sacc);
         pacc = M::mfma32(da, vb, pacc);
       }
+      // LDS reads two k-steps (eight fragments) ahead of the MFMAs that use them
+      __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+#pragma unroll
+      for (int i = 0; i < 2 * C::KSTEPS - 4; i++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
 
       // ---- P and dS -----------------------------------------------------------
       const bool full = iw0 + 31 < len_q && jw1 < len_k &&
@@ -268,6 +295,10 @@ __global__ __launch_bounds__(512) void attn_bwd_dkdv_kernel(const AttnArgs a) {
       }
 
       // ---- dV^T += dO^T P ; dK^T += Q^T dS --------------------------------------
+      // P and dS are packed to 16 bits before the matrix section starts, which leaves
+      // the registers for LDS reads in flight: transposing reads run four fragments
+      // (eight reads) ahead of their MFMA
+      V8 pb[2], dsb[2];
 #pragma unroll
       for (int ks = 0; ks < 2; ks++) {
         float pv[8], dsv[8];
@@ -276,16 +307,27 @@ __global__ __launch_bounds__(512) void attn_bwd_dkdv_kernel(const AttnArgs a) {
           pv[j] = sacc[8 * ks + j];
           dsv[j] = pacc[8 * ks + j];
         }
-        const V8 pb = M::pack(pv);
-        const V8 dsb = M::pack(dsv);
+        pb[ks] = M::pack(pv);
+        dsb[ks] = M::pack(dsv);
+        asm volatile("" : "+v"(pb[ks]), "+v"(dsb[ks]));
+      }
+#pragma unroll
+      for (int ks = 0; ks < 2; ks++) {
 #pragma unroll
         for (int d = 0; d < C::DBLK; d++) {
           const int off0 = (t_row0 ^ (d << 6)) + ks * 16 * C::ROWB;
           const int off1 = (t_row1 ^ (d << 6)) + ks * 16 * C::ROWB;
-          dv_acc[d] = M::mfma32(tr_pair<V8>(do_lds + off0, do_lds + off1), pb, dv_acc[d]);
-          dk_acc[d] = M::mfma32(tr_pair<V8>(q_lds + off0, q_lds + off1), dsb, dk_acc[d]);
+          dv_acc[d] = M::mfma32(tr_pair<V8>(do_lds + off0, do_lds + off1), pb[ks], dv_acc[d]);
+          dk_acc[d] = M::mfma32(tr_pair<V8>(q_lds + off0, q_lds + off1), dsb[ks], dk_acc[d]);
         }
       }
+      __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+#pragma unroll
+      for (int i = 0; i < 4 * C::DBLK - 4; i++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
     }
     __syncthreads();
   };
@@ -360,7 +402,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(const AttnArgs a) {
   if (wid < 0) return;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31;
   const int g = lane >> 5;
   const int i16 = lane & 15;
@@ -489,6 +531,14 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(const AttnArgs a) {
           pacc[t] = M::mfma32(*(const V8*)(vc + off + t * 32 * C::ROWB), dof[ks], pacc[t]);
         }
       }
+      // LDS reads eight fragments ahead of the MFMAs that use them
+      __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+#pragma unroll
+      for (int i = 0; i < 4 * C::KSTEPS - 8; i++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
       const bool full = wave_rows_full && j1 <= wb_first.hi &&
                         (j0 >= wb_last.lo || j1 < a.n_sink);
       if (full) {
@@ -513,20 +563,33 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(const AttnArgs a) {
             pacc[t][i] = ok ? p * (pacc[t][i] - delta) : 0.f;
           }
       }
-      // dQ^T[d, query] += K^T dS^T
+      // dQ^T[d, query] += K^T dS^T; dS^T is packed before the matrix section starts and the
+      // transposing reads run four fragments ahead of their MFMA
+      V8 dsb[4];
 #pragma unroll
       for (int s4 = 0; s4 < 4; s4++) {
         float dsv[8];
 #pragma unroll
         for (int j = 0; j < 8; j++) dsv[j] = pacc[s4 >> 1][8 * (s4 & 1) + j];
-        const V8 dsb = M::pack(dsv);
+        dsb[s4] = M::pack(dsv);
+        asm volatile("" : "+v"(dsb[s4]));
+      }
+#pragma unroll
+      for (int s4 = 0; s4 < 4; s4++) {
 #pragma unroll
         for (int d = 0; d < C::DBLK; d++) {
           const int off0 = (t_row0 ^ (d << 6)) + s4 * 16 * C::ROWB;
           const int off1 = (t_row1 ^ (d << 6)) + s4 * 16 * C::ROWB;
-          dq_acc[d] = M::mfma32(tr_pair<V8>(kc + off0, kc + off1), dsb, dq_acc[d]);
+          dq_acc[d] = M::mfma32(tr_pair<V8>(kc + off0, kc + off1), dsb[s4], dq_acc[d]);
         }
       }
+      __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+#pragma unroll
+      for (int i = 0; i < 4 * C::DBLK - 4; i++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
     }
     __syncthreads();
   };

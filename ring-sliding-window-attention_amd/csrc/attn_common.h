@@ -202,7 +202,7 @@ struct TileDma {
   int wave;
   __device__ __forceinline__ void init(int64_t stride_elems, int tid) {
     const int lane = tid & 63;
-    wave = tid >> 6;
+    wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 #pragma unroll
     for (int n = 0; n < N; n++) {
       const int row = (n * NW + wave) * RPI + lane / CPR;
