@@ -26,6 +26,12 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBPS = 8000.0     # MI355X HBM3E
+# HBM bytes per launch (read + written) of the two roofline kernels at the shapes timed below,
+# from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --pmc-pass`, each counter
+# scaled by what it reads for the 1 GiB device copy of that pass (FETCH_SIZE x2.0, WRITE_SIZE
+# x1.0); the summary is profiles/c3_own_chunk_kernels_hbm_traffic_pmc.txt.
+DKDV_HBM_BYTES_PER_LAUNCH = 738.7e6
+MERGE_HBM_BYTES_PER_LAUNCH = 5693.2e6
 
 
 def band_pairs(length: int, w: int) -> int:
@@ -109,6 +115,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the per-kernel / merge extras")
+    ap.add_argument("--pmc-pass", action="store_true",
+                    help="counter-collection pass: launch a 1 GiB device copy (the known-size "
+                         "calibration kernel) and every hot kernel twice, then exit")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build covers the single-GPU path only; run with --gpus 1 "
@@ -146,6 +155,25 @@ def main():
         out = ring_swa.ring_rank_share_attn(q, k, v, [prev], W, CP, RANK)
         out.backward(do)
 
+    if args.pmc_pass:
+        with torch.no_grad():
+            src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+            dst = torch.empty_like(src)
+            qd, kd, vd = q.detach(), k.detach(), v.detach()
+            dq, dk, dv = torch.empty_like(qd), torch.empty_like(kd), torch.empty_like(vd)
+            acc = torch.randn(1, 131072, HQ, D, device=dev)
+            lacc = torch.randn(1, HQ, 131072, device=dev, dtype=torch.float64)
+            new = torch.randn(1, 131072, HQ, D, device=dev, dtype=torch.bfloat16)
+            lnew = torch.randn(1, HQ, 131072, device=dev)
+            for _ in range(2):
+                dst.copy_(src)  # reads 1 GiB, writes 1 GiB
+                o_d, lse_d = attn_fwd(qd, kd, vd, None, (W, 0), True)
+                attn_bwd(qd, kd, vd, o_d, lse_d, do, dq, dk, dv, None, (W, 0), True)
+                merge_attn_out(acc, lacc, new, lnew)
+            torch.cuda.synchronize()
+        print(json.dumps({"pmc_pass": "done", "copy_bytes_each_way": 1 << 30}))
+        return
+
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -181,39 +209,49 @@ def main():
     }
 
     # ---- roofline of the dominant kernel: backward dK/dV kernel, own-chunk block ----
+    # Algorithmic FLOPs per visible (query, key) pair and q head: forward 4 D (S, PV);
+    # dK/dV kernel 8 D (S, dP, dV, dK); dQ kernel 6 D (S, dP, dQ); the backward as a whole
+    # is credited 10 D (S and dP counted once), as in the headline metric.
     with torch.no_grad():
         qd, kd, vd = q.detach(), k.detach(), v.detach()
         o_d, lse_d = attn_fwd(qd, kd, vd, None, (W, 0), True)
         dq, dk, dv = torch.empty_like(qd), torch.empty_like(kd), torch.empty_like(vd)
-        from ring_swa import _lib
-        ws = torch.empty(int(64 + qd.numel() * 4 + qd.numel() // D * 4 + 4096), dtype=torch.uint8,
-                         device=dev)
+        ws = torch.empty(S * HQ * 8 + 4096, dtype=torch.uint8, device=dev)
         bwd = lambda ph: attn_bwd(qd, kd, vd, o_d, lse_d, do, dq, dk, dv, None, (W, 0), True,  # noqa: E731
                                   workspace=ws, phases=ph)
         bwd(7)
         n = 5 if args.no_extras else 20
-        main_med, main_avg = event_ms(lambda: bwd(2), n)
-        fl_main = 10 * D * pairs_diag * HQ
+        PREP, DKDV, DQ = 1, 2, 4
+        dkdv_med, dkdv_avg = event_ms(lambda: bwd(DKDV), n)
+        fl_pair = D * pairs_diag * HQ
         rec["roofline"] = {
-            "kernel": "attn_bwd_kernel<bf16,128> (own-chunk block 8192x8192, window 4096)",
+            "kernel": "attn_bwd_dkdv_kernel<bf16,128> (own-chunk block 8192x8192, window 4096)",
             "bound": "mfma",
-            "achieved": fl_main / (main_avg * 1e-3) / 1e12,
+            "achieved": 8 * fl_pair / (dkdv_avg * 1e-3) / 1e12,
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
-            "frac": fl_main / (main_avg * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
-            "traffic": None,
-            "avg_launch_ms": main_avg,
-            "median_launch_ms": main_med,
-            "flops_per_launch": fl_main,
+            "frac": 8 * fl_pair / (dkdv_avg * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+            "traffic": DKDV_HBM_BYTES_PER_LAUNCH,
+            "avg_launch_ms": dkdv_avg,
+            "median_launch_ms": dkdv_med,
+            "flops_per_launch": 8 * fl_pair,
         }
         if not args.no_extras:
             fwd_med, _ = event_ms(lambda: attn_fwd(qd, kd, vd, None, (W, 0), True), 20)
+            dq_med, _ = event_ms(lambda: bwd(DQ), 20)
+            prep_med, _ = event_ms(lambda: bwd(PREP), 20)
             bwd_med, _ = event_ms(lambda: bwd(7), 20)
-            fl_fwd = 4 * D * pairs_diag * HQ
+            tf = lambda fl, ms_: fl / ms_ / 1e9  # noqa: E731
             rec["kernels"] = {
-                "fwd_own_chunk": {"ms": fwd_med, "TFLOP/s": fl_fwd / fwd_med / 1e9},
-                "bwd_own_chunk_all_phases": {"ms": bwd_med, "TFLOP/s": fl_main / bwd_med / 1e9},
-                "bwd_own_chunk_main_kernel": {"ms": main_med, "TFLOP/s": fl_main / main_med / 1e9},
+                "fwd_own_chunk": {"ms": fwd_med, "TFLOP/s": tf(4 * fl_pair, fwd_med),
+                                  "flops_per_pair": "4 D"},
+                "bwd_dkdv_own_chunk": {"ms": dkdv_med, "TFLOP/s": tf(8 * fl_pair, dkdv_med),
+                                       "flops_per_pair": "8 D"},
+                "bwd_dq_own_chunk": {"ms": dq_med, "TFLOP/s": tf(6 * fl_pair, dq_med),
+                                     "flops_per_pair": "6 D"},
+                "bwd_prep_own_chunk": {"ms": prep_med},
+                "bwd_own_chunk_all_kernels": {"ms": bwd_med, "TFLOP/s": tf(10 * fl_pair, bwd_med),
+                                              "flops_per_pair": "10 D (window-effective)"},
             }
             # config 2: plain single-GPU SWA, batch 2, seq 8192, 32/32 heads, window 1000
             q2, k2, v2, do2 = (mk(2, 8192, 32, 128) for _ in range(4))
@@ -242,7 +280,8 @@ def main():
                     rec["roofline_merge"] = {
                         "kernel": "merge_kernel<float,bf16,16>", "bound": "hbm",
                         "achieved": nbytes / avg / 1e6, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
-                        "frac": nbytes / avg / 1e6 / PEAK_HBM_GBPS, "traffic": None,
+                        "frac": nbytes / avg / 1e6 / PEAK_HBM_GBPS,
+                        "traffic": MERGE_HBM_BYTES_PER_LAUNCH,
                         "avg_launch_ms": avg, "bytes_per_launch": nbytes}
                 del acc, lacc, new, lnew
             rec["merge"] = merges

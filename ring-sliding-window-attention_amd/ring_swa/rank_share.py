@@ -142,63 +142,89 @@ class RankShareVarlenFunc(torch.autograd.Function):
                 None, None, None, *dprev)
 
 
+_SIDE_STREAMS = {}
+
+
+def _fork(device: torch.device) -> "torch.cuda.Stream":
+    """Side stream (default priority, one per device) ordered after the current stream.
+
+    The blocks of one step are independent until they are merged, and each launch alone
+    leaves compute units idle in its tail (few, unequal work groups), so the diagonal
+    block runs on the caller's stream and the other blocks on this one; ``_join``
+    orders the caller's stream after them again."""
+    side = _SIDE_STREAMS.get(device.index)
+    if side is None:
+        side = _SIDE_STREAMS[device.index] = torch.cuda.Stream(device)
+    side.wait_stream(torch.cuda.current_stream(device))
+    return side
+
+
+def _join(side: "torch.cuda.Stream", device: torch.device) -> None:
+    torch.cuda.current_stream(device).wait_stream(side)
+
+
 def _forward_blocks(q, k, v, prev_kv, plan, scale, local_cu, ring_dtypes):
     """Run the planned blocks and merge them.  Dense 4-d tensors (batch 1 when packed)."""
-    b, s, hq, d = q.shape
-    out = lse = None
+    assert plan and plan[0][0] == 0, "the diagonal block comes first: it covers every row"
+    side = _fork(q.device) if len(plan) > 1 else None
+    parts = []
     for (i, qs, ks, window, causal) in plan:
-        kk, vv = (k, v) if i == 0 else (prev_kv[i - 1][0], prev_kv[i - 1][1])
-        if i == 0 and local_cu is not None:
-            o_i, l_i = attn_fwd(q[0], kk[0], vv[0], scale, window, causal, local_cu, local_cu)
-            o_i, l_i = o_i.unsqueeze(0), l_i.unsqueeze(0)
-        else:
-            o_i, l_i = attn_fwd(q[:, qs], kk[:, ks], vv[:, ks], scale, window, causal)
-        if out is None:
-            # the diagonal block covers every row: it seeds the accumulators directly
-            assert i == 0
-            if ring_dtypes:
-                # accumulator types of ring_swa/sliding_window/nonvarlen.py:53-59
-                out, lse = o_i.float(), l_i.double()
+        if i == 0:
+            if local_cu is not None:
+                o_i, l_i = attn_fwd(q[0], k[0], v[0], scale, window, causal, local_cu, local_cu)
+                o_i, l_i = o_i.unsqueeze(0), l_i.unsqueeze(0)
             else:
-                out, lse = o_i, l_i
+                o_i, l_i = attn_fwd(q, k, v, scale, window, causal)
         else:
-            merge_attn_out(out[:, qs], lse[:, :, qs], o_i, l_i)
+            kk, vv = prev_kv[i - 1][0], prev_kv[i - 1][1]
+            with torch.cuda.stream(side):
+                o_i, l_i = attn_fwd(q[:, qs], kk[:, ks], vv[:, ks], scale, window, causal)
+        parts.append((qs, o_i, l_i))
+    if side is not None:
+        _join(side, q.device)
+    _, out, lse = parts[0]
+    if ring_dtypes:
+        # accumulator types of ring_swa/sliding_window/nonvarlen.py:53-59
+        out, lse = out.float(), lse.double()
+    for qs, o_i, l_i in parts[1:]:
+        merge_attn_out(out[:, qs], lse[:, :, qs], o_i, l_i)
     return out.to(q.dtype), lse.float()
 
 
 def _backward_blocks(q, k, v, prev_kv, out, lse, do, plan, scale, local_cu):
     if do.stride(-1) != 1:
         do = do.contiguous()
+    assert plan and plan[0][0] == 0
     single = len(plan) == 1
-    dq_acc = None if single else torch.zeros_like(q, dtype=torch.float32)
-    dq = dk = dv = None
-    dprev = [None] * len(prev_kv)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    dprev = [torch.zeros_like(kv) for kv in prev_kv]
+    # every buffer is allocated on the caller's stream before the fork
+    dq_parts = [(qs, torch.empty_like(q[:, qs])) for (i, qs, _, _, _) in plan if i > 0]
+    side = None if single else _fork(q.device)
+    n = 0
     for (i, qs, ks, window, causal) in plan:
-        kk, vv = (k, v) if i == 0 else (prev_kv[i - 1][0], prev_kv[i - 1][1])
         if i == 0:
-            dq_i, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
             if local_cu is not None:
-                attn_bwd(q[0], kk[0], vv[0], out[0], lse[0], do[0], dq_i[0], dk[0], dv[0], scale,
+                attn_bwd(q[0], k[0], v[0], out[0], lse[0], do[0], dq[0], dk[0], dv[0], scale,
                          window, causal, local_cu, local_cu)
             else:
-                attn_bwd(q, kk, vv, out, lse, do, dq_i, dk, dv, scale, window, causal)
-            if single:
-                dq = dq_i
-            else:
-                dq_acc.add_(dq_i)
+                attn_bwd(q, k, v, out, lse, do, dq, dk, dv, scale, window, causal)
         else:
             # rows / keys outside the slices receive nothing from this block
-            dkv = torch.zeros_like(prev_kv[i - 1])
-            dq_i = torch.empty_like(q[:, qs])
-            attn_bwd(q[:, qs], kk[:, ks], vv[:, ks], out[:, qs], lse[:, :, qs], do[:, qs], dq_i,
-                     dkv[0][:, ks], dkv[1][:, ks], scale, window, causal)
-            dq_acc[:, qs].add_(dq_i)
-            dprev[i - 1] = dkv
+            kk, vv = prev_kv[i - 1][0], prev_kv[i - 1][1]
+            dkv = dprev[i - 1]
+            with torch.cuda.stream(side):
+                attn_bwd(q[:, qs], kk[:, ks], vv[:, ks], out[:, qs], lse[:, :, qs], do[:, qs],
+                         dq_parts[n][1], dkv[0][:, ks], dkv[1][:, ks], scale, window, causal)
+            n += 1
     if not single:
+        _join(side, q.device)
+        # dq accumulates in fp32 across the blocks, as upstream does
+        # (ring_swa/sliding_window/nonvarlen.py:203, 318-321)
+        dq_acc = dq.float()
+        for qs, dq_i in dq_parts:
+            dq_acc[:, qs].add_(dq_i)
         dq = dq_acc.to(q.dtype)
-    for n, g in enumerate(dprev):
-        if g is None:
-            dprev[n] = torch.zeros_like(prev_kv[n])
     return (dq, dk, dv, *dprev)
 
 
