@@ -48,6 +48,7 @@ def window_allowed(
     window: Tuple[int, int] = (-1, -1),
     causal: bool = False,
     n_sink: int = 0,
+    device=None,
 ) -> torch.Tensor:
     """Boolean ``[sq, sk]`` matrix, True where query row i may see key j.
 
@@ -60,10 +61,10 @@ def window_allowed(
     wl, wr = window
     if causal:
         wr = 0
-    i = torch.arange(sq).unsqueeze(1)
-    j = torch.arange(sk).unsqueeze(0)
+    i = torch.arange(sq, device=device).unsqueeze(1)
+    j = torch.arange(sk, device=device).unsqueeze(0)
     rel = j - i - (sk - sq)
-    ok = torch.ones(sq, sk, dtype=torch.bool)
+    ok = torch.ones(sq, sk, dtype=torch.bool, device=device)
     if wl >= 0:
         ok &= rel >= -wl
     if wr >= 0:
@@ -163,7 +164,7 @@ def window_attention(
     Restates ``ring_swa/ops/wrap_flash.py:168-200`` (what it returns) through
     the closed form of ``test/test_local_swa.py:51-93``.
     """
-    allowed = window_allowed(q.shape[1], k.shape[1], window, causal, n_sink)
+    allowed = window_allowed(q.shape[1], k.shape[1], window, causal, n_sink, device=q.device)
     return masked_attention(q, k, v, allowed, softmax_scale, compute_dtype)
 
 
