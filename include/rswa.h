@@ -154,6 +154,12 @@ typedef struct rswa_attn_params {
   int64_t dv_stride[3];
   void* workspace;        /* >= rswa_attn_bwd_workspace_bytes(), 256-byte aligned */
   uint64_t workspace_bytes;
+  /* != 0: dq += this call's dQ instead of dq = (the buffer's 16-bit values and the new
+   * 16-bit values are added in fp32 and rounded once: what the reference's fp32 dq
+   * accumulator over two ring blocks gives, ring_swa/sliding_window/nonvarlen.py:318-321,
+   * without the extra passes over dq).  dk / dv are always overwritten. */
+  int32_t dq_accumulate;
+  int32_t reserved_;
 } rswa_attn_params;
 
 int rswa_attn_fwd(const rswa_attn_params* p, void* stream);

@@ -102,6 +102,7 @@ int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a) {
   a.n_sink = p->num_sink;
   a.shift_explicit = p->shift_explicit != 0;
   a.shift_val = p->shift;
+  a.dq_accumulate = backward && p->dq_accumulate != 0;
   a.n_tile = 0;
   a.n_work = 0;
   a.scale = p->softmax_scale;

@@ -622,8 +622,16 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(const AttnArgs a) {
         const int c = lane + n * 64;
         const int row = c / C::CPR, col = (c % C::CPR) * 8;
         if (r0 + row < len_q) {
-          const u32x4 val = *(const u32x4*)(stage + row * C::O_STRIDE + col * 2);
-          *(u32x4*)(dq_ptr + (int64_t)(r0 + row) * a.dq_st[1] + col) = val;
+          V8 val = *(const V8*)(stage + row * C::O_STRIDE + col * 2);
+          T* dst = dq_ptr + (int64_t)(r0 + row) * a.dq_st[1] + col;
+          if (a.dq_accumulate) {
+            const V8 old = *(const V8*)dst;
+            float sum[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) sum[j] = (float)old[j] + (float)val[j];
+            val = M::pack(sum);
+          }
+          *(V8*)dst = val;
         }
       }
     }

@@ -70,6 +70,8 @@ class AttnParams(Structure):
         ("dv_stride", _I64x3),
         ("workspace", c_void_p),
         ("workspace_bytes", c_uint64),
+        ("dq_accumulate", c_int32),
+        ("reserved_", c_int32),
     ]
 
 

@@ -143,12 +143,15 @@ def attn_bwd(
     mask_shift: Optional[int] = None,
     workspace: Optional[torch.Tensor] = None,
     phases: int = 7,
+    dq_accumulate: bool = False,
 ) -> None:
     """Masked attention backward; overwrites ``dq, dk, dv`` (views are fine).
 
-    ``workspace`` (uint8, at least ``rswa_attn_bwd_workspace_bytes``) may be supplied to
-    avoid the per-call scratch allocation; ``phases`` is the bit mask of
-    ``rswa_attn_bwd_phases`` (1 prep, 2 dk/dv kernel, 4 dq kernel) for profiling."""
+    ``workspace`` (uint8, at least ``bwd_workspace_bytes(q)``) may be supplied to avoid the
+    per-call scratch allocation, and must be when the phases of one backward are spread
+    over several calls; ``phases`` is the bit mask of ``rswa_attn_bwd_phases`` (1 prep,
+    2 dk/dv kernel, 4 dq kernel).  ``dq_accumulate`` adds this call's dQ to the values
+    already in ``dq`` (fp32 add of the two 16-bit values, one rounding)."""
     packed = cu_seqlens_q is not None
     _check_qkv(q, k, v, packed)
     dev = _lib.require_device(q, k, v, o, softmax_lse, do, dq, dk, dv)
@@ -168,12 +171,14 @@ def attn_bwd(
     if softmax_scale is None:
         softmax_scale = q.shape[-1] ** (-0.5)
     if q.numel() == 0 or k.numel() == 0:
-        dq.zero_()
+        if not dq_accumulate:
+            dq.zero_()
         dk.zero_()
         dv.zero_()
         return
     p = _params(q, k, v, softmax_scale, window_size, causal, cu_seqlens_q, cu_seqlens_k, num_sink,
                 mask_shift)
+    p.dq_accumulate = int(bool(dq_accumulate))
     p.out = o.data_ptr()
     p.out_stride = _lib.i64x3(_strides3(o, packed))
     p.lse = softmax_lse.data_ptr()
@@ -193,6 +198,13 @@ def attn_bwd(
     p.workspace_bytes = workspace.numel()
     with torch.cuda.device(dev):
         _lib.check(L.rswa_attn_bwd_phases(p, _lib.stream_ptr(dev), int(phases)))
+
+
+def bwd_workspace_bytes(q: torch.Tensor) -> int:
+    """Scratch size of one backward over the rows of ``q`` (dense ``[B,S,H,D]`` or packed
+    ``[T,H,D]``): two fp32 values per (row, head), as ``rswa_attn_bwd_workspace_bytes``
+    computes it, plus alignment slack."""
+    return (q.numel() // q.shape[-1]) * 8 + 1024
 
 
 # ---- names of the upstream wrappers -----------------------------------------

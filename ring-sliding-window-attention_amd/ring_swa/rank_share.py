@@ -19,7 +19,7 @@ from typing import List, Optional, Sequence, Tuple
 
 import torch
 
-from .ops.band_attn import attn_bwd, attn_fwd
+from .ops.band_attn import attn_bwd, attn_fwd, bwd_workspace_bytes
 from .ops.lse_merge import merge_attn_out
 
 Step = Tuple[int, slice, slice, Tuple[int, int], bool]
@@ -195,6 +195,8 @@ def _backward_blocks(q, k, v, prev_kv, out, lse, do, plan, scale, local_cu):
     if do.stride(-1) != 1:
         do = do.contiguous()
     assert plan and plan[0][0] == 0
+    if len(plan) == 2:
+        return _backward_two_blocks(q, k, v, prev_kv, out, lse, do, plan, scale, local_cu)
     single = len(plan) == 1
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     dprev = [torch.zeros_like(kv) for kv in prev_kv]
@@ -225,6 +227,39 @@ def _backward_blocks(q, k, v, prev_kv, out, lse, do, plan, scale, local_cu):
         for qs, dq_i in dq_parts:
             dq_acc[:, qs].add_(dq_i)
         dq = dq_acc.to(q.dtype)
+    return (dq, dk, dv, *dprev)
+
+
+def _backward_two_blocks(q, k, v, prev_kv, out, lse, do, plan, scale, local_cu):
+    """Own-chunk block + one previous-chunk block (window no longer than a chunk): dq is
+    summed inside the dQ kernel instead of in separate passes.  The previous-chunk block
+    writes its dQ first (side stream, onto zeros); the own-chunk dQ kernel, ordered after
+    it, adds to it: fp32 sum of the two 16-bit partials, rounded once -- bit for bit what
+    the fp32 accumulator of ring_swa/sliding_window/nonvarlen.py:203, 318-321 yields for two
+    blocks.  The own-chunk dK/dV kernel is independent of all that and overlaps it."""
+    PREP, DKDV, DQ = 1, 2, 4
+    (_, _, _, window0, causal0), (i1, qs, ks, window1, causal1) = plan
+    dq, dk, dv = torch.zeros_like(q), torch.empty_like(k), torch.empty_like(v)
+    dprev = [torch.zeros_like(kv) for kv in prev_kv]
+    ws = torch.empty(bwd_workspace_bytes(q), dtype=torch.uint8, device=q.device)
+
+    def own(phases, accumulate):
+        if local_cu is not None:
+            attn_bwd(q[0], k[0], v[0], out[0], lse[0], do[0], dq[0], dk[0], dv[0], scale, window0,
+                     causal0, local_cu, local_cu, workspace=ws, phases=phases,
+                     dq_accumulate=accumulate)
+        else:
+            attn_bwd(q, k, v, out, lse, do, dq, dk, dv, scale, window0, causal0, workspace=ws,
+                     phases=phases, dq_accumulate=accumulate)
+
+    side = _fork(q.device)
+    own(PREP | DKDV, False)
+    kk, vv, dkv = prev_kv[i1 - 1][0], prev_kv[i1 - 1][1], dprev[i1 - 1]
+    with torch.cuda.stream(side):
+        attn_bwd(q[:, qs], kk[:, ks], vv[:, ks], out[:, qs], lse[:, :, qs], do[:, qs], dq[:, qs],
+                 dkv[0][:, ks], dkv[1][:, ks], scale, window1, causal1, dq_accumulate=True)
+    _join(side, q.device)
+    own(DQ, True)
     return (dq, dk, dv, *dprev)
 
 

@@ -228,3 +228,29 @@ def test_bwd_fp16():
     _, _, gq, gk, gv = _run_dense(q, k, v, do, 0.2, (33, 0), True, 0)
     errs = [_relnorm(g, r) for g, r in ((gq, rq), (gk, rk), (gv, rv))]
     assert max(errs) <= GRAD_TOL, f"rel-norm errors dq/dk/dv = {errs}"
+
+
+@pytest.mark.parametrize("hq,hk,s", [(4, 2, 300), (3, 3, 257)])
+def test_bwd_dq_accumulate_is_one_fp32_add_of_the_two_16bit_values(hq, hk, s):
+    """dq_accumulate: dq <- round(float(dq) + float(round(dQ))), bit for bit; dk / dv as
+    without it.  Also with the phases of one backward spread over two calls, as the
+    two-block ring step uses them."""
+    from ring_swa.ops import attn_bwd, attn_fwd
+    from ring_swa.ops.band_attn import bwd_workspace_bytes
+
+    g = torch.Generator().manual_seed(7)
+    q, do = (torch.randn(2, s, hq, 128, generator=g).bfloat16().cuda() for _ in range(2))
+    k, v = (torch.randn(2, s, hk, 128, generator=g).bfloat16().cuda() for _ in range(2))
+    base = torch.randn(2, s, hq, 128, generator=g).bfloat16().cuda()
+    out, lse = attn_fwd(q, k, v, None, (100, 0), True)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    attn_bwd(q, k, v, out, lse, do, dq, dk, dv, None, (100, 0), True)
+    acc, dk2, dv2 = base.clone(), torch.empty_like(k), torch.empty_like(v)
+    ws = torch.empty(bwd_workspace_bytes(q), dtype=torch.uint8, device="cuda")
+    attn_bwd(q, k, v, out, lse, do, acc, dk2, dv2, None, (100, 0), True, workspace=ws, phases=3)
+    assert torch.equal(acc, base)  # the dQ kernel has not run yet
+    attn_bwd(q, k, v, out, lse, do, acc, dk2, dv2, None, (100, 0), True, workspace=ws, phases=4,
+             dq_accumulate=True)
+    torch.cuda.synchronize()
+    assert torch.equal(acc, (base.float() + dq.float()).bfloat16())
+    assert torch.equal(dk2, dk) and torch.equal(dv2, dv)
