@@ -224,49 +224,6 @@ struct TileDma {
   }
 };
 
-// Byte offset of a __shared__ object inside the block's LDS allocation.
-__device__ __forceinline__ unsigned lds_offset(const void* p) {
-  return (unsigned)(uintptr_t)(lds_void_t*)p;
-}
-
-// The same tile copy issued through inline assembly.  The compiler then does not know
-// that LDS is written, so it inserts no wait before LDS reads that follow (it cannot
-// prove, for dynamically indexed tile buffers, that they do not alias the load); the
-// caller orders the accesses itself with wait_dma() and a block barrier.  M0 carries the
-// LDS destination; nothing else in these kernels uses M0 (gfx9 LDS instructions do not
-// read it), so it is not saved.
-template <int D, int ROWS, int THREADS>
-struct TileDmaAsm {
-  static constexpr int CPR = D / 8;
-  static constexpr int RPI = 64 / CPR;
-  static constexpr int NW = THREADS / 64;
-  static constexpr int N = ROWS * CPR / THREADS;
-  static_assert(N >= 1 && N * THREADS == ROWS * CPR, "tile must divide evenly");
-  static_assert((NW * RPI) % 16 == 0, "row step must preserve the swizzle");
-  int voff;
-  int step_bytes;
-  int wave;
-  __device__ __forceinline__ void init(int64_t stride_elems, int tid) {
-    const int lane = tid & 63;
-    wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int row = wave * RPI + lane / CPR;
-    voff = (int)(row * stride_elems * 2) + (((lane % CPR) ^ swz_f<CPR>(row)) << 4);
-    step_bytes = (int)(NW * RPI * stride_elems * 2);
-  }
-  __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t rsrc, int soff,
-                                       unsigned lds_tile) const {
-#pragma unroll
-    for (int n = 0; n < N; n++) {
-      const unsigned dst = lds_tile + (n * NW + wave) * 1024;
-      const int so = soff + n * step_bytes;
-      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                   :
-                   : "s"(dst), "v"(voff), "s"(rsrc), "s"(so)
-                   : "memory");
-    }
-  }
-};
-
 // Block barrier that waits for this wave's LDS traffic only: loads still in flight from
 // global memory into LDS (vmcnt) are NOT drained, unlike __syncthreads().  A wave that
 // issued such loads calls wait_dma() before the barrier that publishes them.
