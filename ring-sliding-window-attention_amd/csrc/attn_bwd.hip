@@ -150,6 +150,9 @@ __global__ __launch_bounds__(512) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   const T* q_base = (const T*)a.q + b * a.q_st[0] + s.q_row0 * a.q_st[1];
   const T* do_base = (const T*)a.dout + b * a.do_st[0] + s.q_row0 * a.do_st[1];
   const int q_row_bytes = (int)(a.q_st[1] * 2), do_row_bytes = (int)(a.do_st[1] * 2);
+  // bytes from a head's first row to the end of its last row (see make_rows_rsrc)
+  const int q_extent = (len_q - 1) * q_row_bytes + C::ROWB;
+  const int do_extent = (len_q - 1) * do_row_bytes + C::ROWB;
   // statistics: one resource over both workspace arrays (lse2 then delta); rows past the
   // sequence end read a neighbour's finite values, which the row mask / zero Q, dO rows void
   const int64_t stat_elems = a.delta - a.lse2;  // elements between the two arrays
@@ -172,16 +175,22 @@ __global__ __launch_bounds__(512) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   nxt.do_head = do_base + (int64_t)hk * a.group * a.do_st[2];
   nxt.stat_row = (int64_t)hk * a.group * a.rows_q + ws_row0;
   auto load_next = [&](char* qd, char* dod, float* std_) __attribute__((always_inline)) {
-    const __amdgpu_buffer_rsrc_t q_rsrc = make_rows_rsrc(nxt.q_head, len_q, a.q_st[1] * 2, C::ROWB);
+    const __amdgpu_buffer_rsrc_t q_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void*)nxt.q_head, 0, q_extent, 0x00020000);
     const __amdgpu_buffer_rsrc_t do_rsrc =
-        make_rows_rsrc(nxt.do_head, len_q, a.do_st[1] * 2, C::ROWB);
-    q_dma.load(q_rsrc, nxt.i0 * q_row_bytes, qd);
-    do_dma.load(do_rsrc, nxt.i0 * do_row_bytes, dod);
+        __builtin_amdgcn_make_buffer_rsrc((void*)nxt.do_head, 0, do_extent, 0x00020000);
     if (wave < 2) {  // wave 0: lse2 tile, wave 1: delta tile (64 floats each)
       const int soff = (int)((nxt.stat_row + nxt.i0 + wave * stat_elems) * 4);
+      // the per-lane offset is recomputed here (opaque to the optimiser): kept in a
+      // register across the walk it gets spilled, and its reload would wait for every
+      // tile load issued before it
+      int lane4 = lane;
+      asm volatile("v_lshlrev_b32 %0, 2, %0" : "+v"(lane4));
       __builtin_amdgcn_raw_ptr_buffer_load_lds(st_rsrc, (lds_void_t*)(std_ + wave * C::BM), 4,
-                                               lane * 4, soff, 0, 0);
+                                               lane4, soff, 0, 0);
     }
+    q_dma.load(q_rsrc, nxt.i0 * q_row_bytes, qd);
+    do_dma.load(do_rsrc, nxt.i0 * do_row_bytes, dod);
     nxt.qt++;
     nxt.i0 += C::BM;
     if (nxt.qt == n_qt) {
@@ -206,6 +215,21 @@ __global__ __launch_bounds__(512) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   const char* v_lds = v_s + wk * 32 * C::ROWB;
 
   int cur_i0 = i_first;  // first row of the tile being computed
+  // For which first rows iw0 of a 32-row half-tile does any (query, key of this wave) pair
+  // survive the mask (need_*), and for which is no pair masked (full_*)?  With
+  // iw1 = min(iw0 + 32, len_q) - 1 the conditions
+  //   needed: iw0 < len_q, jw0 < len_k, jw0 <= iw1 + shift + wr, (jw1 >= iw0 + shift - wl or sink)
+  //   full:   iw0 + 31 < len_q, jw1 < len_k, jw1 <= iw0 + shift + wr,
+  //           (jw0 >= iw0 + 31 + shift - wl or all 32 keys are sinks)
+  // are intervals of iw0 whose ends depend on the wave only: a step tests two of them.
+  const int jw1 = jw0 + 31;
+  constexpr int kInf = 1 << 30;
+  int need_lo = (a.wr < 0) ? -kInf : jw0 - shift - a.wr - 31;
+  int need_hi = min(len_q - 1, (a.wl < 0 || jw0 < a.n_sink) ? kInf : jw1 - shift + a.wl);
+  if (jw0 >= len_k || (a.wr >= 0 && len_q - 1 < jw0 - shift - a.wr)) need_hi = -kInf - 1;
+  int full_lo = (a.wr < 0) ? -kInf : jw1 - shift - a.wr;
+  int full_hi = min(len_q - 32, (a.wl < 0 || jw1 < a.n_sink) ? kInf : jw0 - 31 - shift + a.wl);
+  if (jw1 >= len_k) full_hi = -kInf - 1;
   // one query tile: prefetch the next one into (qn, don, stn), compute on (qc, doc, stc)
   auto step = [&](int it, const char* qc, const char* doc, const float* stc, char* qn, char* don,
                   float* stn) __attribute__((always_inline)) {
@@ -217,117 +241,119 @@ __global__ __launch_bounds__(512) void attn_bwd_dkdv_kernel(const AttnArgs a) {
     const float* lse_lds = stc + wq * 32;
     const float* delta_lds = lse_lds + C::BM;
 
-    // Does any (query of this wave's half-tile, key of this wave) pair survive the mask?
     const int iw0 = i0 + wq * 32;
-    const int iw1 = min(iw0 + 32, len_q) - 1;
-    const int jw1 = jw0 + 31;
-    const bool needed = iw0 < len_q && jw0 < len_k &&
-                        (a.wr < 0 || jw0 <= iw1 + shift + a.wr) &&
-                        (a.wl < 0 || jw1 >= iw0 + shift - a.wl || jw0 < a.n_sink);
+    const bool needed = iw0 >= need_lo && iw0 <= need_hi;
     if (needed) {
-      // ---- S = Q K^T and dP = dO V^T (rows = queries, lane = key column) ------
+      const bool full = iw0 >= full_lo && iw0 <= full_hi;
+      // key position relative to the aligned diagonal of row iw0: rel(r) = rel0 - r
+      const int rel0 = jc - iw0 - shift;
+      const int rel_hi = (a.wr < 0) ? (1 << 30) : a.wr;
+      const int rel_lo = (a.wl < 0 || jc < a.n_sink) ? -(1 << 30) : -a.wl;
+      const int rows_ok = (jc < len_k) ? len_q - iw0 : 0;  // rows r < rows_ok are real
+
+      // The 4 GEMMs of the sub-tile (S, dP, dV, dK: KS MFMAs each), their LDS reads and
+      // the vector work are written out in issue order, one group per MFMA, with
+      // scheduling fences between the groups: fragments are read four MFMAs ahead,
+      // P = exp2(S c - lse2) is computed under the dP MFMAs and dS = P (dP - delta) under
+      // the dV MFMAs, so that the matrix pipe never waits for the vector ALU.
+      constexpr int KS = C::KSTEPS;  // MFMAs per GEMM (= 2 DBLK)
+      constexpr int AHEAD = 3;
+      static_assert(KS == 2 * C::DBLK && KS >= AHEAD, "GEMM shapes");
+      auto fence = []() __attribute__((always_inline)) { __builtin_amdgcn_sched_barrier(0); };
+      V8 fa[4 * KS], fb[2 * KS];  // A fragments of MFMA 0 .. 4 KS - 1, B fragments of S and dP
+      auto fetch = [&](int m) __attribute__((always_inline)) {
+        if (m < KS) {
+          const int off = a_row ^ (m << 5);
+          fa[m] = *(const V8*)(q_lds + off);
+          fb[m] = *(const V8*)(k_lds + off);
+        } else if (m < 2 * KS) {
+          const int off = a_row ^ ((m - KS) << 5);
+          fa[m] = *(const V8*)(do_lds + off);
+          fb[m] = *(const V8*)(v_lds + off);
+        } else if (m < 4 * KS) {
+          const int j = (m - 2 * KS) % KS, ks = j / C::DBLK, d = j % C::DBLK;
+          const char* src = m < 3 * KS ? do_lds : q_lds;
+          const int off0 = (t_row0 ^ (d << 6)) + ks * 16 * C::ROWB;
+          const int off1 = (t_row1 ^ (d << 6)) + ks * 16 * C::ROWB;
+          fa[m] = tr_pair<V8>(src + off0, src + off1);
+        }
+      };
       f32x16 sacc, pacc;
 #pragma unroll
       for (int i = 0; i < 16; i++) {
         sacc[i] = 0.f;
         pacc[i] = 0.f;
       }
+      f32x4 l4[4], d4[4];
+      V8 pb[2], dsb[2];
+      // vector work, in four chunks of four rows each
+      auto p_chunk = [&](int c) __attribute__((always_inline)) {
 #pragma unroll
-      for (int ks = 0; ks < C::KSTEPS; ks++) {
-        const int off = a_row ^ (ks << 5);
-        const V8 qa = *(const V8*)(q_lds + off);
-        const V8 kb = *(const V8*)(k_lds + off);
-        const V8 da = *(const V8*)(do_lds + off);
-        const V8 vb = *(const V8*)(v_lds + off);
-        sacc = M::mfma32(qa, kb, sacc);
-        pacc = M::mfma32(da, vb, pacc);
-      }
-      // LDS reads two k-steps (eight fragments) ahead of the MFMAs that use them
-      __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
-#pragma unroll
-      for (int i = 0; i < 2 * C::KSTEPS - 4; i++) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-      }
-      __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
-
-      // ---- P and dS -----------------------------------------------------------
-      const bool full = iw0 + 31 < len_q && jw1 < len_k &&
-                        (a.wr < 0 || jw1 <= iw0 + shift + a.wr) &&
-                        (a.wl < 0 || jw0 >= iw0 + 31 + shift - a.wl || jw1 < a.n_sink);
-      if (full) {
-#pragma unroll
-        for (int i4 = 0; i4 < 4; i4++) {
-          const int rbase = 8 * i4 + 4 * g;
-          const f32x4 l4 = *(const f32x4*)(lse_lds + rbase);
-          const f32x4 d4 = *(const f32x4*)(delta_lds + rbase);
-#pragma unroll
-          for (int e = 0; e < 4; e++) {
-            const int i = 4 * i4 + e;
-            const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[i], a.scale_log2, -l4[e]));
-            sacc[i] = p;
-            pacc[i] = p * (pacc[i] - d4[e]);
-          }
+        for (int e = 0; e < 4; e++) {
+          const int i = 4 * c + e;
+          sacc[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[i], a.scale_log2, -l4[c][e]));
         }
-      } else {
-        // key position relative to the aligned diagonal of row iw0: rel(r) = rel0 - r
-        const int rel0 = jc - iw0 - shift;
-        const int rel_hi = (a.wr < 0) ? (1 << 30) : a.wr;
-        const int rel_lo = (a.wl < 0 || jc < a.n_sink) ? -(1 << 30) : -a.wl;
-        const int rows_ok = (jc < len_k) ? len_q - iw0 : 0;  // rows r < rows_ok are real
-#pragma unroll
-        for (int i4 = 0; i4 < 4; i4++) {
-          const int rbase = 8 * i4 + 4 * g;
-          const f32x4 l4 = *(const f32x4*)(lse_lds + rbase);
-          const f32x4 d4 = *(const f32x4*)(delta_lds + rbase);
+        if (!full) {
 #pragma unroll
           for (int e = 0; e < 4; e++) {
-            const int i = 4 * i4 + e;
-            const int r = rbase + e;
+            const int r = 8 * c + 4 * g + e;
             const int rel = rel0 - r;
             const bool ok = (r < rows_ok) & (rel <= rel_hi) & (rel >= rel_lo);
-            float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[i], a.scale_log2, -l4[e]));
-            p = ok ? p : 0.f;
-            sacc[i] = p;
-            pacc[i] = ok ? p * (pacc[i] - d4[e]) : 0.f;
+            sacc[4 * c + e] = ok ? sacc[4 * c + e] : 0.f;
           }
         }
-      }
+        if (c & 1) {
+          float pv[8];
+#pragma unroll
+          for (int j = 0; j < 8; j++) pv[j] = sacc[8 * (c >> 1) + j];
+          pb[c >> 1] = M::pack(pv);
+        }
+      };
+      auto ds_chunk = [&](int c) __attribute__((always_inline)) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const int i = 4 * c + e;
+          pacc[i] = sacc[i] * (pacc[i] - d4[c][e]);  // zero wherever P was masked to zero
+        }
+        if (c & 1) {
+          float dsv[8];
+#pragma unroll
+          for (int j = 0; j < 8; j++) dsv[j] = pacc[8 * (c >> 1) + j];
+          dsb[c >> 1] = M::pack(dsv);
+        }
+      };
 
-      // ---- dV^T += dO^T P ; dK^T += Q^T dS --------------------------------------
-      // P and dS are packed to 16 bits before the matrix section starts, which leaves
-      // the registers for LDS reads in flight: transposing reads run four fragments
-      // (eight reads) ahead of their MFMA
-      V8 pb[2], dsb[2];
 #pragma unroll
-      for (int ks = 0; ks < 2; ks++) {
-        float pv[8], dsv[8];
+      for (int m = 0; m < AHEAD; m++) fetch(m);
+      fence();
 #pragma unroll
-        for (int j = 0; j < 8; j++) {
-          pv[j] = sacc[8 * ks + j];
-          dsv[j] = pacc[8 * ks + j];
+      for (int m = 0; m < 4 * KS; m++) {
+        fetch(m + AHEAD);
+        // row statistics of chunk c: read two groups before the chunk that uses them
+        {
+          constexpr int LAG = KS > 4 ? 1 : 0;  // chunk c runs in group KS + c + LAG (2 KS + ...)
+          const int cl = m - (KS + LAG - 2), cd = m - (2 * KS + LAG - 2);
+          if (cl >= 0 && cl < 4) l4[cl] = *(const f32x4*)(lse_lds + 8 * cl + 4 * g);
+          if (cd >= 0 && cd < 4) d4[cd] = *(const f32x4*)(delta_lds + 8 * cd + 4 * g);
         }
-        pb[ks] = M::pack(pv);
-        dsb[ks] = M::pack(dsv);
-        asm volatile("" : "+v"(pb[ks]), "+v"(dsb[ks]));
-      }
-#pragma unroll
-      for (int ks = 0; ks < 2; ks++) {
-#pragma unroll
-        for (int d = 0; d < C::DBLK; d++) {
-          const int off0 = (t_row0 ^ (d << 6)) + ks * 16 * C::ROWB;
-          const int off1 = (t_row1 ^ (d << 6)) + ks * 16 * C::ROWB;
-          dv_acc[d] = M::mfma32(tr_pair<V8>(do_lds + off0, do_lds + off1), pb[ks], dv_acc[d]);
-          dk_acc[d] = M::mfma32(tr_pair<V8>(q_lds + off0, q_lds + off1), dsb[ks], dk_acc[d]);
+        if (m < KS) {
+          sacc = M::mfma32(fa[m], fb[m], sacc);
+        } else if (m < 2 * KS) {
+          pacc = M::mfma32(fa[m], fb[m], pacc);
+          // P chunks under dP MFMAs 1 .. 4 (D = 128) / 0 .. 3 (D = 64)
+          const int c = m - KS - (KS > 4 ? 1 : 0);
+          if (c >= 0 && c < 4) p_chunk(c);
+        } else if (m < 3 * KS) {
+          const int j = m - 2 * KS;
+          dv_acc[j % C::DBLK] = M::mfma32(fa[m], pb[j / C::DBLK], dv_acc[j % C::DBLK]);
+          const int c = j - (KS > 4 ? 1 : 0);
+          if (c >= 0 && c < 4) ds_chunk(c);
+        } else {
+          const int j = m - 3 * KS;
+          dk_acc[j % C::DBLK] = M::mfma32(fa[m], dsb[j / C::DBLK], dk_acc[j % C::DBLK]);
         }
+        fence();
       }
-      __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
-#pragma unroll
-      for (int i = 0; i < 4 * C::DBLK - 4; i++) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-      }
-      __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
     }
     __syncthreads();
   };
