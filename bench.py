@@ -284,6 +284,18 @@ def main():
                         "traffic": MERGE_HBM_BYTES_PER_LAUNCH,
                         "avg_launch_ms": avg, "bytes_per_launch": nbytes}
                 del acc, lacc, new, lnew
+            # the reference's merge-only sweep (ring_swa/ops/merge.py:257-302): B 1, H 32, D 128
+            sweep = {}
+            for rows_s in (1024, 4096, 16384, 65536, 131072):
+                acc = torch.randn(1, rows_s, HQ, D, device=dev)
+                lacc = torch.randn(1, HQ, rows_s, device=dev, dtype=torch.float64)
+                new = torch.randn(1, rows_s, HQ, D, device=dev, dtype=torch.bfloat16)
+                lnew = torch.randn(1, HQ, rows_s, device=dev)
+                med, _ = event_ms(lambda: merge_attn_out(acc, lacc, new, lnew), 20)
+                sweep[f"s{rows_s}"] = {"us": med * 1e3,
+                                       "GB/s": rows_s * HQ * (10 * D + 20) / med / 1e6}
+                del acc, lacc, new, lnew
+            merges["sweep_ring_dtypes"] = sweep
             rec["merge"] = merges
             rec["merge_GBps"] = merges["sweep_s131072"]["GB/s"]
 

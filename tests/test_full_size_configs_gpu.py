@@ -34,11 +34,25 @@ def _rel(x, ref):
     return ((x - ref).norm() / ref.norm().clamp_min(1e-30)).item()
 
 
+def _mismatch_fraction(x, ref, atol=2.5e-2, rtol=2.5e-2):
+    """The reference's own acceptance rule (test/test_ring_swa_nonvarlen.py:196-229):
+    share of elements outside atol + rtol * |ref|."""
+    bad = (x.float() - ref).abs() > atol + rtol * ref.abs()
+    return bad.float().mean().item()
+
+
 def _check(name, out, grads, ref_out, ref_grads):
     err = (out.float() - ref_out).abs().max().item()
     assert err <= OUT_TOL, f"{name}: out max-abs {err}"
     errs = [_rel(g, r) for g, r in zip(grads, ref_grads)]
     assert max(errs) <= GRAD_TOL, f"{name}: rel-norm dq/dk/dv = {errs}"
+    # secondary, in the reference's style.  The reference asks for fewer than 0.01 % of the
+    # elements off on unscaled N(0,1) inputs; the output meets that everywhere, and so do
+    # the gradients except with the x4 sink keys of configuration 5, where gradients are
+    # several times larger and about 0.02 % of dq end up past the bound (P and dS enter the
+    # MFMAs as 16-bit values); 0.05 % is asserted for gradients.
+    fr = [_mismatch_fraction(a, b) for a, b in zip((out, *grads), (ref_out, *ref_grads))]
+    assert fr[0] < 1e-4 and max(fr) < 5e-4, f"{name}: mismatched fraction out/dq/dk/dv = {fr}"
 
 
 def test_config2_swa_batch2_seq8192_mha_window1000():
@@ -155,22 +169,29 @@ def test_config4_varlen_rank_slices_total32768_window2048():
         assert torch.isfinite(t.float()).all()
 
 
-@pytest.mark.parametrize("impl", ["split", "fused"])
-def test_config5_streaming_llm_varlen_total65536_4sinks(impl):
+@pytest.mark.parametrize("impl,n_sink", [("split", 4), ("fused", 4), ("split", 1)])
+def test_config5_streaming_llm_varlen_total65536_sinks(impl, n_sink):
+    """n_sink = 4: the configuration as stated (keyword-only extension of the API);
+    n_sink = 1: the reference's own single sink through the unchanged signature."""
     import ring_swa
 
-    total, hq, hk, n_sink, w = 65536, 32, 8, 4, 4092
+    total, hq, hk, w = 65536, 32, 8, 4092
     g = torch.Generator().manual_seed(0)
     cuts = sorted((torch.randperm(total // 1024 - 1, generator=g)[:3] + 1).tolist())
     cu = [0] + [c * 1024 for c in cuts] + [total]
     q, do = _randn((total, hq, D), 0), _randn((total, hq, D), 1)
     k, v = _randn((total, hk, D), 2), _randn((total, hk, D), 3)
     for c in cu[:-1]:
-        k[c:c + n_sink] *= 4  # peaked softmax mass on the sink keys
+        # every sequence starts with the same sink rows (the reference's precondition,
+        # test/test_ring_slm_varlen.py:145-147), keys scaled for peaked softmax mass
+        for t in (q, k, v):
+            t[c:c + n_sink] = t[:n_sink]
+    for c in cu[:-1]:
+        k[c:c + n_sink] *= 4
     cu_dev = torch.tensor(cu, dtype=torch.int32, device="cuda")
     qg, kg, vg = (t.clone().requires_grad_() for t in (q, k, v))
-    out = ring_swa.ring_streaming_llm_attn_varlen(qg, kg, vg, w, cu_dev, cp_size=1,
-                                                  num_sink_tokens=n_sink, impl=impl)
+    kw = {} if n_sink == 1 else {"num_sink_tokens": n_sink}
+    out = ring_swa.ring_streaming_llm_attn_varlen(qg, kg, vg, w, cu_dev, cp_size=1, impl=impl, **kw)
     out.backward(do)
     gq, gk = slice(0, hq // hk), slice(0, 1)
     # the oracle one sequence at a time (score matrices of the longest sequence: GBs)
