@@ -15,9 +15,9 @@
 // directly in LDS, issued one (V) and two (K) tiles ahead.  The buffers are SEPARATE
 // static __shared__ arrays and the tile loop is unrolled by two, so that every access
 // names its buffer statically: only then can the compiler tell that an in-flight load
-// does not alias the LDS reads of the current tile, and not wait for it.  Inside a wave
-// the loop is software-pipelined: the QK^T MFMAs of tile t+1 are issued together with
-// the softmax (vector ALU) of tile t, so the matrix and vector pipes overlap.
+// does not alias the LDS reads of the current tile, and not wait for it.  The two waves
+// of a SIMD run half a tile apart (ping-pong, see the tile loop): the softmax of one is
+// executed under the MFMAs of the other.
 #include "attn_common.h"
 
 namespace rswa {
