@@ -111,6 +111,22 @@ class RankShareFunc(torch.autograd.Function):
         return (grads[0], grads[1], grads[2], None, None, None, None, None, *grads[3:])
 
 
+_CU_CACHE = {}
+
+
+def _device_cu(local_cu: Sequence[int], device: torch.device) -> torch.Tensor:
+    """int32 device copy of a rank's local ``cu_seqlens``, cached: a training loop calls
+    every layer with the same packing, and each fresh host-to-device copy of a Python list
+    is a blocking call that stops the host from running ahead of the GPU."""
+    key = (tuple(local_cu), device.index)
+    t = _CU_CACHE.get(key)
+    if t is None:
+        if len(_CU_CACHE) >= 256:
+            _CU_CACHE.clear()
+        t = _CU_CACHE[key] = torch.tensor(local_cu, dtype=torch.int32, device=device)
+    return t
+
+
 class RankShareVarlenFunc(torch.autograd.Function):
     """Packed tensors ``[tokens, heads, dim]``; ``prev_kv[i - 1]`` is ``[2, tokens, kv_heads, dim]``."""
 
@@ -121,7 +137,7 @@ class RankShareVarlenFunc(torch.autograd.Function):
         if softmax_scale is None:
             softmax_scale = d ** (-0.5)
         local_cu, plan = plan_varlen(cu_host, s, window_size, cp_size, rank)
-        cu_dev = torch.tensor(local_cu, dtype=torch.int32, device=q.device)
+        cu_dev = _device_cu(local_cu, q.device)
         q4, k4, v4 = q.unsqueeze(0), k.unsqueeze(0), v.unsqueeze(0)
         prev4 = [p.unsqueeze(1) for p in prev_kv]
         out, lse = _forward_blocks(q4, k4, v4, prev4, plan, softmax_scale, cu_dev, ring_dtypes)
