@@ -4,11 +4,11 @@
 // Three launches on the caller's stream:
 //   PREP : per (row, q head): delta = sum_d dO * O and lse2 = lse * log2(e) (-inf -> +inf),
 //          both fp32, into the caller's workspace
-//   DKDV : one block (8 waves) owns 128 keys of one (sequence, kv head), keeps their K and
-//          V tiles in LDS and walks the query tiles (64 rows) that can see them, for every
-//          q head of the GQA group; wave (wk, wq) handles key columns 32 wk.. of query rows
-//          32 wq.. of each tile; dK^T / dV^T partials stay in registers for the whole walk,
-//          the two query halves are added through LDS at the end and written once
+//   DKDV : one block (4 waves, one per SIMD, up to 512 registers each) owns 256 keys of one
+//          (sequence, kv head) and walks the query tiles (32 rows) that can see them, for
+//          every q head of the GQA group; a wave owns 64 keys: their K fragments stay in
+//          registers, their V rows in LDS, dK^T / dV^T accumulate in accumulation registers
+//          for the whole walk and are written once
 //   DQ   : one block (8 waves x 32 query rows: 128 rows of two q heads of a GQA group, or
 //          256 rows of one head) walks the key tiles (64 keys) it can see, like the forward
 //          kernel; dQ^T stays in registers
@@ -17,18 +17,23 @@
 // channel, which caps an atomic dQ far below the MFMA rate.  It also makes the result
 // run-to-run deterministic.
 //
-// DKDV per (query half-tile, wave) (C layout: lane = key):
-//   S = Q K^T, dP = dO V^T      A = Q / dO row fragments, B = K / V row fragments (all LDS)
+// DKDV per (query tile, wave) (C layout: lane = key; two 32-key blocks per wave, so every
+// fragment read from LDS feeds two MFMAs):
+//   S = Q K^T, dP = dO V^T      A = Q / dO row fragments (LDS), B = K (registers) / V (LDS)
 //   P = exp2(S*c - lse2), dS = P * (dP - delta)
 //   dV^T += dO^T P, dK^T += Q^T dS   A = transposing LDS reads of dO / Q, B = P / dS (regs)
+// Its MFMAs are inline assembly so that the register file of each accumulator can be
+// chosen: S and dP in vector registers (the vector ALU reads them next), dK^T and dV^T in
+// accumulation registers.  Left to the compiler, S and dP end up in accumulation registers
+// too and every element costs two copies.
 // DQ per (key tile, wave); wave owns 32 query columns (C layout: lane = query):
 //   S^T = K Q^T, dP^T = V dO^T  A = K / V row fragments from LDS, B = Q / dO fragments (regs)
 //   dS^T as above with per-lane lse2 / delta
 //   dQ^T += K^T dS^T            A = transposing LDS reads of K, B = dS^T (regs)
 //
-// Tiles are double-buffered in SEPARATE static __shared__ arrays, filled by buffer loads
-// that land directly in LDS one tile ahead, and the tile loops are unrolled by two so that
-// every access names its buffer statically (see attn_fwd.hip for why).
+// Streamed tiles are double-buffered in SEPARATE static __shared__ arrays, filled by buffer
+// loads that land directly in LDS one tile ahead, and the tile loops are unrolled by two so
+// that every access names its buffer statically (see attn_fwd.hip for why).
 #include "attn_common.h"
 
 namespace rswa {
@@ -39,29 +44,25 @@ namespace {
 // ============================================================================
 template <int D>
 struct DkvCfg {
-  static constexpr int BM = 64;        // query rows per step
-  static constexpr int BN = 128;       // keys per block
-  static constexpr int THREADS = 512;  // 8 waves: 4 key groups x 2 query halves
+  static constexpr int BM = 32;        // query rows per step
+  static constexpr int KB = 2;         // 32-key blocks per wave
+  static constexpr int BN = 256;       // keys per block: 4 waves x KB x 32
+  static constexpr int THREADS = 256;  // one wave per SIMD, up to 512 registers each
   static constexpr int KSTEPS = D / 16;
   static constexpr int DBLK = D / 32;
   static constexpr int CPR = D / 8;   // 16-byte chunks per row
   static constexpr int ROWB = D * 2;  // bytes per row
   static constexpr int Q_TILE = BM * ROWB;
-  static constexpr int KV_TILE = BN * ROWB;
-  // end-of-walk reduction of the two query halves, one matrix (dK, then dV) at a time:
-  // per key group DBLK x 16 registers x 64 lanes fp32, staged in the K tile (key groups
-  // 0-1) and the V tile (key groups 2-3)
-  static constexpr int RED_PER_WK = DBLK * 16 * 64 * 4;
-  static_assert(2 * RED_PER_WK <= KV_TILE, "reduction staging must fit the K and V tiles");
+  static constexpr int V_TILE = BN * ROWB;
 };
 
 template <typename T, int D>
-__global__ __launch_bounds__(512) void attn_bwd_dkdv_kernel(const AttnArgs a) {
+__global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   using C = DkvCfg<D>;
   using M = Mma<T>;
   using V8 = typename M::V8;
-  __shared__ __attribute__((aligned(1024))) char k_s[C::KV_TILE];
-  __shared__ __attribute__((aligned(1024))) char v_s[C::KV_TILE];
+  constexpr int KB = C::KB, KS = C::KSTEPS, DB = C::DBLK;
+  __shared__ __attribute__((aligned(1024))) char v_s[C::V_TILE];
   __shared__ __attribute__((aligned(1024))) char q_s0[C::Q_TILE];
   __shared__ __attribute__((aligned(1024))) char q_s1[C::Q_TILE];
   __shared__ __attribute__((aligned(1024))) char do_s0[C::Q_TILE];
@@ -73,9 +74,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   if (wid < 0) return;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wk = wave & 3;   // key group: columns 32 wk .. 32 wk + 31 of the block's 128 keys
-  const int wq = wave >> 2;  // query half: rows 32 wq .. 32 wq + 31 of each 64-row tile
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // key group: 64 keys each
   const int l32 = lane & 31;
   const int g = lane >> 5;
   const int i16 = lane & 15;
@@ -117,21 +116,12 @@ __global__ __launch_bounds__(512) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   const int n_qt = (i_max >= i_min) ? i_max / C::BM - qt_lo + 1 : 0;
   const int n_iter = n_qt * a.group;
 
-  const int jw0 = j0 + wk * 32;  // first key column of this wave
-  const int jc = jw0 + l32;      // this lane's key column
-
-  f32x16 dk_acc[C::DBLK], dv_acc[C::DBLK];
-#pragma unroll
-  for (int d = 0; d < C::DBLK; d++)
-#pragma unroll
-    for (int i = 0; i < 16; i++) {
-      dk_acc[d][i] = 0.f;
-      dv_acc[d][i] = 0.f;
-    }
+  const int jw0 = j0 + wave * (32 * KB);  // first key column of this wave
+  const int jw1 = jw0 + 32 * KB - 1;
 
   // ---- lane-constant LDS offsets (swizzle folded: varying parts are XOR / immediates) ----
-  // 16-byte row fragments: row = 32 blk + l32, chunk = 2 ks + g
-  //   offset = (a_row ^ (ks << 5)) + blk * 32 * ROWB      (Q / dO: blk = wq; K / V: blk = wk)
+  // 16-byte row fragments: row = l32 (+ 32 per block), chunk = 2 ks + g
+  //   offset = (a_row ^ (ks << 5)) + blk * 32 * ROWB
   const int a_row = l32 * C::ROWB + ((g ^ swz_f<C::CPR>(l32)) << 4);
   // transposing reads of Q / dO: rows 16 ks + 4 g + (i16 >> 2) and + 8, chunk = 4 d + lp
   //   offset = (t_row{0,1} ^ (d << 6)) + ks * 16 * ROWB
@@ -140,10 +130,36 @@ __global__ __launch_bounds__(512) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   const int t_row0 = rl * C::ROWB + ((lp ^ swz_f<C::CPR>(rl)) << 4) + (i16 & 1) * 8;
   const int t_row1 = (rl + 8) * C::ROWB + ((lp ^ swz_f<C::CPR>(rl + 8)) << 4) + (i16 & 1) * 8;
 
+  // ---- this wave's K fragments stay in registers for the whole walk (B operand of
+  // S = Q K^T: lane = key column, 8 consecutive d per k-step); keys past the end are zero
+  V8 kf[KB][KS];
+#pragma unroll
+  for (int kb = 0; kb < KB; kb++) {
+    const int jc = jw0 + kb * 32 + l32;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      if (jc < len_k) {
+        kf[kb][ks] = *(const V8*)(k_ptr + (int64_t)jc * a.k_st[1] + ks * 16 + g * 8);
+      } else {
+        kf[kb][ks] = V8{0, 0, 0, 0, 0, 0, 0, 0};
+      }
+    }
+  }
+
+  f32x16 dk_acc[KB][DB], dv_acc[KB][DB];
+#pragma unroll
+  for (int kb = 0; kb < KB; kb++)
+#pragma unroll
+    for (int d = 0; d < DB; d++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        dk_acc[kb][d][i] = 0.f;
+        dv_acc[kb][d][i] = 0.f;
+      }
+
   // ---- tile DMA (rows past the end of the sequence read as zero) ------------------
-  TileDma<D, C::BN, C::THREADS> k_dma, v_dma;
+  TileDma<D, C::BN, C::THREADS> v_dma;
   TileDma<D, C::BM, C::THREADS> q_dma, do_dma;
-  k_dma.init(a.k_st[1], tid);
   v_dma.init(a.v_st[1], tid);
   q_dma.init(a.q_st[1], tid);
   do_dma.init(a.do_st[1], tid);
@@ -168,29 +184,39 @@ __global__ __launch_bounds__(512) void attn_bwd_dkdv_kernel(const AttnArgs a) {
     int64_t stat_row;  // index of row 0 of this head in the statistics arrays
   };
   const int i_first = qt_lo * C::BM;
-  Cursor nxt;  // the tile that load_next() fetches
+  Cursor nxt;  // the tile that the load parts fetch
   nxt.qt = 0;
   nxt.i0 = i_first;
   nxt.q_head = q_base + (int64_t)hk * a.group * a.q_st[2];
   nxt.do_head = do_base + (int64_t)hk * a.group * a.do_st[2];
   nxt.stat_row = (int64_t)hk * a.group * a.rows_q + ws_row0;
-  auto load_next = [&](char* qd, char* dod, float* std_) __attribute__((always_inline)) {
-    const __amdgpu_buffer_rsrc_t q_rsrc =
-        __builtin_amdgcn_make_buffer_rsrc((void*)nxt.q_head, 0, q_extent, 0x00020000);
-    const __amdgpu_buffer_rsrc_t do_rsrc =
-        __builtin_amdgcn_make_buffer_rsrc((void*)nxt.do_head, 0, do_extent, 0x00020000);
-    if (wave < 2) {  // wave 0: lse2 tile, wave 1: delta tile (64 floats each)
-      const int soff = (int)((nxt.stat_row + nxt.i0 + wave * stat_elems) * 4);
-      // the per-lane offset is recomputed here (opaque to the optimiser): kept in a
-      // register across the walk it gets spilled, and its reload would wait for every
-      // tile load issued before it
-      int lane4 = lane;
-      asm volatile("v_lshlrev_b32 %0, 2, %0" : "+v"(lane4));
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(st_rsrc, (lds_void_t*)(std_ + wave * C::BM), 4,
-                                               lane4, soff, 0, 0);
+  // The next tile is fetched by NPART instructions per wave (statistics, Q, dO), issued
+  // one at a time between the first MFMAs of a step; advance() then moves the cursor on.
+  constexpr int NQD = TileDma<D, C::BM, C::THREADS>::N;
+  constexpr int NPART = 1 + 2 * NQD;
+  auto load_part = [&](int part, char* qd, char* dod, float* std_) __attribute__((always_inline)) {
+    if (part == 0) {
+      if (wave == 0) {  // lanes 0-31: lse2 of the 32 rows, lanes 32-63: their delta
+        const int soff = (int)((nxt.stat_row + nxt.i0) * 4);
+        // the per-lane offset is recomputed here (opaque to the optimiser): kept in a
+        // register across the walk it could be spilled, and its reload would wait for
+        // every tile load issued before it
+        int l = lane;
+        asm volatile("" : "+v"(l));
+        const int voff = ((l & 31) << 2) + (l >> 5) * (int)(stat_elems * 4);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(st_rsrc, (lds_void_t*)std_, 4, voff, soff, 0, 0);
+      }
+    } else if (part <= NQD) {
+      const __amdgpu_buffer_rsrc_t q_rsrc =
+          __builtin_amdgcn_make_buffer_rsrc((void*)nxt.q_head, 0, q_extent, 0x00020000);
+      q_dma.load_one(q_rsrc, nxt.i0 * q_row_bytes, qd, part - 1);
+    } else {
+      const __amdgpu_buffer_rsrc_t do_rsrc =
+          __builtin_amdgcn_make_buffer_rsrc((void*)nxt.do_head, 0, do_extent, 0x00020000);
+      do_dma.load_one(do_rsrc, nxt.i0 * do_row_bytes, dod, part - 1 - NQD);
     }
-    q_dma.load(q_rsrc, nxt.i0 * q_row_bytes, qd);
-    do_dma.load(do_rsrc, nxt.i0 * do_row_bytes, dod);
+  };
+  auto advance = [&]() __attribute__((always_inline)) {
     nxt.qt++;
     nxt.i0 += C::BM;
     if (nxt.qt == n_qt) {
@@ -203,26 +229,24 @@ __global__ __launch_bounds__(512) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   };
 
   if (n_iter > 0) {
-    const __amdgpu_buffer_rsrc_t k_rsrc = make_rows_rsrc(k_ptr, len_k, a.k_st[1] * 2, C::ROWB);
     const __amdgpu_buffer_rsrc_t v_rsrc = make_rows_rsrc(v_ptr, len_k, a.v_st[1] * 2, C::ROWB);
-    k_dma.load(k_rsrc, (int)(j0 * a.k_st[1] * 2), k_s);
     v_dma.load(v_rsrc, (int)(j0 * a.v_st[1] * 2), v_s);
-    load_next(q_s0, do_s0, st_s0);
+#pragma unroll
+    for (int part = 0; part < NPART; part++) load_part(part, q_s0, do_s0, st_s0);
+    advance();
   }
   __syncthreads();
 
-  const char* k_lds = k_s + wk * 32 * C::ROWB;
-  const char* v_lds = v_s + wk * 32 * C::ROWB;
+  const char* v_lds = v_s + wave * (32 * KB) * C::ROWB;
 
   int cur_i0 = i_first;  // first row of the tile being computed
-  // For which first rows iw0 of a 32-row half-tile does any (query, key of this wave) pair
-  // survive the mask (need_*), and for which is no pair masked (full_*)?  With
-  // iw1 = min(iw0 + 32, len_q) - 1 the conditions
-  //   needed: iw0 < len_q, jw0 < len_k, jw0 <= iw1 + shift + wr, (jw1 >= iw0 + shift - wl or sink)
-  //   full:   iw0 + 31 < len_q, jw1 < len_k, jw1 <= iw0 + shift + wr,
-  //           (jw0 >= iw0 + 31 + shift - wl or all 32 keys are sinks)
-  // are intervals of iw0 whose ends depend on the wave only: a step tests two of them.
-  const int jw1 = jw0 + 31;
+  // For which first rows i0 of a 32-row tile does any (query, key of this wave) pair survive
+  // the mask (need_*), and for which is no pair masked (full_*)?  With
+  // i1 = min(i0 + 32, len_q) - 1 and the wave's keys jw0 .. jw1 the conditions
+  //   needed: i0 < len_q, jw0 < len_k, jw0 <= i1 + shift + wr, (jw1 >= i0 + shift - wl or sink)
+  //   full:   i0 + 31 < len_q, jw1 < len_k, jw1 <= i0 + shift + wr,
+  //           (jw0 >= i0 + 31 + shift - wl or all the wave's keys are sinks)
+  // are intervals of i0 whose ends depend on the wave only: a step tests two of them.
   constexpr int kInf = 1 << 30;
   int need_lo = (a.wr < 0) ? -kInf : jw0 - shift - a.wr - 31;
   int need_hi = min(len_q - 1, (a.wl < 0 || jw0 < a.n_sink) ? kInf : jw1 - shift + a.wl);
@@ -230,130 +254,143 @@ __global__ __launch_bounds__(512) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   int full_lo = (a.wr < 0) ? -kInf : jw1 - shift - a.wr;
   int full_hi = min(len_q - 32, (a.wl < 0 || jw1 < a.n_sink) ? kInf : jw0 - 31 - shift + a.wl);
   if (jw1 >= len_k) full_hi = -kInf - 1;
+
   // one query tile: prefetch the next one into (qn, don, stn), compute on (qc, doc, stc)
   auto step = [&](int it, const char* qc, const char* doc, const float* stc, char* qn, char* don,
                   float* stn) __attribute__((always_inline)) {
     const int i0 = cur_i0;
     cur_i0 = nxt.i0;  // the tile fetched now is the next step's
-    if (it + 1 < n_iter) load_next(qn, don, stn);
-    const char* q_lds = qc + wq * 32 * C::ROWB;
-    const char* do_lds = doc + wq * 32 * C::ROWB;
-    const float* lse_lds = stc + wq * 32;
-    const float* delta_lds = lse_lds + C::BM;
-
-    const int iw0 = i0 + wq * 32;
-    const bool needed = iw0 >= need_lo && iw0 <= need_hi;
+    const bool has_next = it + 1 < n_iter;
+    const float* lse_lds = stc;
+    const float* delta_lds = stc + C::BM;
+    const bool needed = i0 >= need_lo && i0 <= need_hi;
+    if (!needed && has_next) {
+#pragma unroll
+      for (int part = 0; part < NPART; part++) load_part(part, qn, don, stn);
+      advance();
+    }
     if (needed) {
-      const bool full = iw0 >= full_lo && iw0 <= full_hi;
-      // key position relative to the aligned diagonal of row iw0: rel(r) = rel0 - r
-      const int rel0 = jc - iw0 - shift;
-      const int rel_hi = (a.wr < 0) ? (1 << 30) : a.wr;
-      const int rel_lo = (a.wl < 0 || jc < a.n_sink) ? -(1 << 30) : -a.wl;
-      const int rows_ok = (jc < len_k) ? len_q - iw0 : 0;  // rows r < rows_ok are real
-
-      // The 4 GEMMs of the sub-tile (S, dP, dV, dK: KS MFMAs each), their LDS reads and
-      // the vector work are written out in issue order, one group per MFMA, with
-      // scheduling fences between the groups: fragments are read four MFMAs ahead,
-      // P = exp2(S c - lse2) is computed under the dP MFMAs and dS = P (dP - delta) under
-      // the dV MFMAs, so that the matrix pipe never waits for the vector ALU.
-      constexpr int KS = C::KSTEPS;  // MFMAs per GEMM (= 2 DBLK)
-      constexpr int AHEAD = 3;
-      static_assert(KS == 2 * C::DBLK && KS >= AHEAD, "GEMM shapes");
+      const bool full = i0 >= full_lo && i0 <= full_hi;
+      const int rel_hi = (a.wr < 0) ? kInf : a.wr;
+      // The four GEMMs of the (32 queries x 64 keys) sub-tile -- S = Q K^T, dP = dO V^T,
+      // dV^T += dO^T P, dK^T += Q^T dS; KB KS MFMAs each, rows = queries, lane = key column
+      // -- their LDS reads and the vector work are written out in issue order, one group
+      // per MFMA, with scheduling fences between the groups.  Every fragment read from LDS
+      // feeds the MFMAs of both key blocks; K comes from registers; fragments are fetched
+      // AH fragment slots ahead; P = exp2(S c - lse2) is computed under the dP MFMAs and
+      // dS = P (dP - delta) under the dV MFMAs.
+      constexpr int NG = KB * KS;   // MFMAs per GEMM (KS = 2 DB)
+      constexpr int NF = 4 * KS;    // fragment slots: Q, dO (+ V), dO^T, Q^T; KB MFMAs each
+      constexpr int AH = 2;
+      constexpr int GPC = NG / (4 * KB);  // MFMA groups per chunk of vector work
+      static_assert(KS == 2 * DB && KB == 2, "GEMM shapes");
       auto fence = []() __attribute__((always_inline)) { __builtin_amdgcn_sched_barrier(0); };
-      V8 fa[4 * KS], fb[2 * KS];  // A fragments of MFMA 0 .. 4 KS - 1, B fragments of S and dP
-      auto fetch = [&](int m) __attribute__((always_inline)) {
-        if (m < KS) {
-          const int off = a_row ^ (m << 5);
-          fa[m] = *(const V8*)(q_lds + off);
-          fb[m] = *(const V8*)(k_lds + off);
-        } else if (m < 2 * KS) {
-          const int off = a_row ^ ((m - KS) << 5);
-          fa[m] = *(const V8*)(do_lds + off);
-          fb[m] = *(const V8*)(v_lds + off);
-        } else if (m < 4 * KS) {
-          const int j = (m - 2 * KS) % KS, ks = j / C::DBLK, d = j % C::DBLK;
-          const char* src = m < 3 * KS ? do_lds : q_lds;
-          const int off0 = (t_row0 ^ (d << 6)) + ks * 16 * C::ROWB;
-          const int off1 = (t_row1 ^ (d << 6)) + ks * 16 * C::ROWB;
-          fa[m] = tr_pair<V8>(src + off0, src + off1);
+      V8 fa[NF], fv[KB][KS];
+      auto fetch = [&](auto fc) __attribute__((always_inline)) {
+        constexpr int f = decltype(fc)::value;
+        if constexpr (f < KS) {
+          fa[f] = *(const V8*)(qc + (a_row ^ (f << 5)));
+        } else if constexpr (f < 2 * KS) {
+          constexpr int ks = f - KS;
+          fa[f] = *(const V8*)(doc + (a_row ^ (ks << 5)));
+#pragma unroll
+          for (int kb = 0; kb < KB; kb++)
+            fv[kb][ks] = *(const V8*)(v_lds + (a_row ^ (ks << 5)) + kb * 32 * C::ROWB);
+        } else if constexpr (f < NF) {
+          constexpr int j = (f - 2 * KS) % KS, ks2 = j / DB, d = j % DB;
+          const char* src = f < 3 * KS ? doc : qc;
+          const int off0 = (t_row0 ^ (d << 6)) + ks2 * 16 * C::ROWB;
+          const int off1 = (t_row1 ^ (d << 6)) + ks2 * 16 * C::ROWB;
+          fa[f] = tr_pair<V8>(src + off0, src + off1);
         }
       };
-      f32x16 sacc, pacc;
-#pragma unroll
-      for (int i = 0; i < 16; i++) {
-        sacc[i] = 0.f;
-        pacc[i] = 0.f;
-      }
+      const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f,
+                           0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      f32x16 sacc[KB], pacc[KB];
       f32x4 l4[4], d4[4];
-      V8 pb[2], dsb[2];
-      // vector work, in four chunks of four rows each
-      auto p_chunk = [&](int c) __attribute__((always_inline)) {
+      V8 pb[KB][2], dsb[KB][2];
+      // vector work in 2 KB chunks of four rows: chunk order lets the packed operands of
+      // the first k-step be complete first
+      auto chunk_of = [](int c, int& kb, int& i4) __attribute__((always_inline)) {
+        kb = (c >> 1) & 1;
+        i4 = (c & 1) | ((c >> 2) << 1);
+      };
+      // P stays in vector registers from here to dS (the S / dP accumulators live in
+      // accumulation registers, which the vector ALU reaches only through copies)
+      float pk[KB][16];
+      auto p_chunk = [&](auto cc) __attribute__((always_inline)) {
+        int kb, i4;
+        chunk_of(decltype(cc)::value, kb, i4);
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-          const int i = 4 * c + e;
-          sacc[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[i], a.scale_log2, -l4[c][e]));
+          const int i = 4 * i4 + e;
+          pk[kb][i] =
+              __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][i], a.scale_log2, -l4[i4][e]));
         }
         if (!full) {
+          // key position relative to the aligned diagonal of row i0: rel(r) = rel0 - r
+          const int jc = jw0 + kb * 32 + l32;
+          const int rel0 = jc - i0 - shift;
+          const int rel_lo = (a.wl < 0 || jc < a.n_sink) ? -kInf : -a.wl;
+          const int rows_ok = (jc < len_k) ? len_q - i0 : 0;  // rows r < rows_ok are real
 #pragma unroll
           for (int e = 0; e < 4; e++) {
-            const int r = 8 * c + 4 * g + e;
+            const int r = 8 * i4 + 4 * g + e;
             const int rel = rel0 - r;
             const bool ok = (r < rows_ok) & (rel <= rel_hi) & (rel >= rel_lo);
-            sacc[4 * c + e] = ok ? sacc[4 * c + e] : 0.f;
+            pk[kb][4 * i4 + e] = ok ? pk[kb][4 * i4 + e] : 0.f;
           }
         }
-        if (c & 1) {
-          float pv[8];
-#pragma unroll
-          for (int j = 0; j < 8; j++) pv[j] = sacc[8 * (c >> 1) + j];
-          pb[c >> 1] = M::pack(pv);
-        }
+        if (i4 & 1) pb[kb][i4 >> 1] = M::pack(&pk[kb][8 * (i4 >> 1)]);
       };
-      auto ds_chunk = [&](int c) __attribute__((always_inline)) {
+      float dsk[KB][8];  // dS of the current pair of chunks
+      auto ds_chunk = [&](auto cc) __attribute__((always_inline)) {
+        int kb, i4;
+        chunk_of(decltype(cc)::value, kb, i4);
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-          const int i = 4 * c + e;
-          pacc[i] = sacc[i] * (pacc[i] - d4[c][e]);  // zero wherever P was masked to zero
+          const int i = 4 * i4 + e;
+          dsk[kb][4 * (i4 & 1) + e] = pk[kb][i] * (pacc[kb][i] - d4[i4][e]);  // zero where P is
         }
-        if (c & 1) {
-          float dsv[8];
-#pragma unroll
-          for (int j = 0; j < 8; j++) dsv[j] = pacc[8 * (c >> 1) + j];
-          dsb[c >> 1] = M::pack(dsv);
-        }
+        if (i4 & 1) dsb[kb][i4 >> 1] = M::pack(dsk[kb]);
       };
 
-#pragma unroll
-      for (int m = 0; m < AHEAD; m++) fetch(m);
+      static_for<AH>([&](auto fc) __attribute__((always_inline)) { fetch(fc); });
       fence();
-#pragma unroll
-      for (int m = 0; m < 4 * KS; m++) {
-        fetch(m + AHEAD);
-        // row statistics of chunk c: read two groups before the chunk that uses them
-        {
-          constexpr int LAG = KS > 4 ? 1 : 0;  // chunk c runs in group KS + c + LAG (2 KS + ...)
-          const int cl = m - (KS + LAG - 2), cd = m - (2 * KS + LAG - 2);
-          if (cl >= 0 && cl < 4) l4[cl] = *(const f32x4*)(lse_lds + 8 * cl + 4 * g);
-          if (cd >= 0 && cd < 4) d4[cd] = *(const f32x4*)(delta_lds + 8 * cd + 4 * g);
-        }
-        if (m < KS) {
-          sacc = M::mfma32(fa[m], fb[m], sacc);
-        } else if (m < 2 * KS) {
-          pacc = M::mfma32(fa[m], fb[m], pacc);
-          // P chunks under dP MFMAs 1 .. 4 (D = 128) / 0 .. 3 (D = 64)
-          const int c = m - KS - (KS > 4 ? 1 : 0);
-          if (c >= 0 && c < 4) p_chunk(c);
-        } else if (m < 3 * KS) {
-          const int j = m - 2 * KS;
-          dv_acc[j % C::DBLK] = M::mfma32(fa[m], pb[j / C::DBLK], dv_acc[j % C::DBLK]);
-          const int c = j - (KS > 4 ? 1 : 0);
-          if (c >= 0 && c < 4) ds_chunk(c);
+      static_for<4 * NG>([&](auto mc) __attribute__((always_inline)) {
+        constexpr int m = decltype(mc)::value;
+        constexpr int f = m / KB, kb = m % KB;  // fragment slot and key block of this MFMA
+        if constexpr (kb == 0) fetch(std::integral_constant<int, f + AH>{});
+        if (m < NPART && has_next) load_part(m, qn, don, stn);
+        // row statistics: lse2 at the end of S, delta at the end of dP
+        if constexpr (m >= NG - 4 && m < NG) l4[m - (NG - 4)] = *(const f32x4*)(lse_lds + 8 * (m - (NG - 4)) + 4 * g);
+        if constexpr (m >= 2 * NG - 4 && m < 2 * NG)
+          d4[m - (2 * NG - 4)] = *(const f32x4*)(delta_lds + 8 * (m - (2 * NG - 4)) + 4 * g);
+        if constexpr (m < NG) {
+          if constexpr (f == 0) {
+            M::mfma32_vec0(fa[f], kf[kb][f], sacc[kb]);
+          } else {
+            M::mfma32_vec(fa[f], kf[kb][f], sacc[kb]);
+          }
+        } else if constexpr (m < 2 * NG) {
+          if constexpr (f == KS) {
+            M::mfma32_vec0(fa[f], fv[kb][f - KS], pacc[kb]);
+          } else {
+            M::mfma32_vec(fa[f], fv[kb][f - KS], pacc[kb]);
+          }
+          if constexpr ((m - NG + 1) % GPC == 0) p_chunk(std::integral_constant<int, (m - NG + 1) / GPC - 1>{});
+        } else if constexpr (m < 3 * NG) {
+          constexpr int j = f - 2 * KS, ks2 = j / DB, d = j % DB;
+          M::mfma32_acc(fa[f], pb[kb][ks2], dv_acc[kb][d]);
+          if constexpr ((m - 2 * NG + 1) % GPC == 0)
+            ds_chunk(std::integral_constant<int, (m - 2 * NG + 1) / GPC - 1>{});
         } else {
-          const int j = m - 3 * KS;
-          dk_acc[j % C::DBLK] = M::mfma32(fa[m], dsb[j / C::DBLK], dk_acc[j % C::DBLK]);
+          constexpr int j = f - 3 * KS, ks2 = j / DB, d = j % DB;
+          M::mfma32_acc(fa[f], dsb[kb][ks2], dk_acc[kb][d]);
         }
         fence();
-      }
+      });
+      if (has_next) advance();
     }
     __syncthreads();
   };
@@ -363,38 +400,29 @@ __global__ __launch_bounds__(512) void attn_bwd_dkdv_kernel(const AttnArgs a) {
     if (it + 1 < n_iter) step(it + 1, q_s1, do_s1, st_s1, q_s0, do_s0, st_s0);
   }
 
-  // ---- add the two query halves (through LDS), then write dK, dV --------------------
-  // (C layout: lane = key, regs = d).  Key groups 0-1 stage in the K tile, 2-3 in the V tile.
-  float* red = (float*)((wk < 2 ? k_s : v_s) + (wk & 1) * C::RED_PER_WK);
+  // ---- write dK, dV (C layout: lane = key, regs = d) -----------------------------------
+  // (the MFMAs above are inline assembly: the compiler does not pad the distance between
+  // the last of them and the first read of their results)
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 #pragma unroll
-  for (int m = 0; m < 2; m++) {  // m = 0: dK, m = 1: dV
-    f32x16* acc = m == 0 ? dk_acc : dv_acc;
-    if (wq == 1) {
+  for (int kb = 0; kb < KB; kb++) {
+    const int jc = jw0 + kb * 32 + l32;
+    if (jc < len_k) {
 #pragma unroll
-      for (int d = 0; d < C::DBLK; d++)
+      for (int mtx = 0; mtx < 2; mtx++) {  // 0: dK, 1: dV
+        const float sc = mtx == 0 ? a.scale : 1.f;
+        T* dst = mtx == 0 ? dk_ptr + (int64_t)jc * a.dk_st[1] : dv_ptr + (int64_t)jc * a.dv_st[1];
 #pragma unroll
-        for (int i4 = 0; i4 < 4; i4++) {
-          const f32x4 x = {acc[d][4 * i4], acc[d][4 * i4 + 1], acc[d][4 * i4 + 2],
-                           acc[d][4 * i4 + 3]};
-          *(f32x4*)(red + ((d * 4 + i4) * 64 + lane) * 4) = x;
-        }
+        for (int d = 0; d < DB; d++)
+#pragma unroll
+          for (int i4 = 0; i4 < 4; i4++) {
+            const f32x16& acc = mtx == 0 ? dk_acc[kb][d] : dv_acc[kb][d];
+            const auto h4 = M::pack4(acc[4 * i4] * sc, acc[4 * i4 + 1] * sc, acc[4 * i4 + 2] * sc,
+                                     acc[4 * i4 + 3] * sc);
+            *(typename M::V4*)(dst + d * 32 + 8 * i4 + 4 * g) = h4;
+          }
+      }
     }
-    __syncthreads();
-    if (wq == 0 && jc < len_k) {
-      const float sc = m == 0 ? a.scale : 1.f;
-      T* dst = (m == 0 ? dk_ptr + (int64_t)jc * a.dk_st[1] : dv_ptr + (int64_t)jc * a.dv_st[1]);
-#pragma unroll
-      for (int d = 0; d < C::DBLK; d++)
-#pragma unroll
-        for (int i4 = 0; i4 < 4; i4++) {
-          const f32x4 x = *(const f32x4*)(red + ((d * 4 + i4) * 64 + lane) * 4);
-          const auto h4 = M::pack4((acc[d][4 * i4] + x[0]) * sc, (acc[d][4 * i4 + 1] + x[1]) * sc,
-                                   (acc[d][4 * i4 + 2] + x[2]) * sc,
-                                   (acc[d][4 * i4 + 3] + x[3]) * sc);
-          *(typename M::V4*)(dst + d * 32 + 8 * i4 + 4 * g) = h4;
-        }
-    }
-    __syncthreads();
   }
 }
 

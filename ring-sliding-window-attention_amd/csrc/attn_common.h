@@ -14,6 +14,9 @@
 
 #include "rswa_common.h"
 
+#include <type_traits>
+#include <utility>
+
 namespace rswa {
 
 constexpr float kLog2e = 1.4426950408889634f;
@@ -114,6 +117,18 @@ struct Mma<__bf16> {
   static __device__ __forceinline__ f32x16 mfma32(V8 a, V8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
+  // The same instruction with the accumulator's register file chosen by the caller:
+  // accumulation registers (for accumulators only MFMAs touch) or vector registers (for
+  // accumulators the vector ALU reads next), and a zero-initialising form.
+  static __device__ __forceinline__ void mfma32_acc(V8 a, V8 b, f32x16& c) {
+    asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void mfma32_vec(V8 a, V8 b, f32x16& c) {
+    asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void mfma32_vec0(V8 a, V8 b, f32x16& c) {
+    asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=v"(c) : "v"(a), "v"(b));
+  }
   static __device__ __forceinline__ V8 pack(const float* x) {
     f32x8 f = {x[0], x[1], x[2], x[3], x[4], x[5], x[6], x[7]};
     return __builtin_convertvector(f, V8);
@@ -130,6 +145,15 @@ struct Mma<_Float16> {
   using V4 = f16x4;
   static __device__ __forceinline__ f32x16 mfma32(V8 a, V8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ void mfma32_acc(V8 a, V8 b, f32x16& c) {
+    asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void mfma32_vec(V8 a, V8 b, f32x16& c) {
+    asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void mfma32_vec0(V8 a, V8 b, f32x16& c) {
+    asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=v"(c) : "v"(a), "v"(b));
   }
   static __device__ __forceinline__ V8 pack(const float* x) {
     f32x8 f = {x[0], x[1], x[2], x[3], x[4], x[5], x[6], x[7]};
@@ -214,15 +238,29 @@ struct TileDma {
     step_bytes = (int)(NW * RPI * stride_elems * 2);
   }
   // `soff` = byte offset of the tile's first row inside the resource (wave-uniform)
+  __device__ __forceinline__ void load_one(__amdgpu_buffer_rsrc_t rsrc, int soff, char* lds_tile,
+                                           int n) const {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(
+        rsrc, (lds_void_t*)(lds_tile + (n * NW + wave) * 1024), 16, voff, soff + n * step_bytes, 0,
+        0);
+  }
   __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t rsrc, int soff, char* lds_tile) const {
 #pragma unroll
-    for (int n = 0; n < N; n++) {
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(
-          rsrc, (lds_void_t*)(lds_tile + (n * NW + wave) * 1024), 16, voff, soff + n * step_bytes,
-          0, 0);
-    }
+    for (int n = 0; n < N; n++) load_one(rsrc, soff, lds_tile, n);
   }
 };
+
+// f(integral_constant<int, 0>{}), ..., f(integral_constant<int, N - 1>{}): a loop whose
+// index is a compile-time constant in every iteration (register arrays indexed by it never
+// fall back to dynamic indexing, whatever the unroller thinks of the body's size).
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
 
 // Block barrier that waits for this wave's LDS traffic only: loads still in flight from
 // global memory into LDS (vmcnt) are NOT drained, unlike __syncthreads().  A wave that
