@@ -1,4 +1,5 @@
 // Host-side validation of rswa_attn_params and translation to kernel arguments.
+#include <algorithm>
 #include "attn_common.h"
 
 namespace rswa {
@@ -105,6 +106,27 @@ int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a) {
   a.dq_accumulate = backward && p->dq_accumulate != 0;
   a.n_tile = 0;
   a.n_work = 0;
+  {
+    // Heaviest tiles first: compare the number of keys the first and the last query row
+    // see, and the number of query rows that see the first and the last key (packed
+    // batches: judged on the average sequence; the order affects speed only).
+    const int64_t lq = packed ? std::max<int64_t>(1, p->total_q / std::max(1, p->batch)) : p->seqlen_q;
+    const int64_t lk = packed ? std::max<int64_t>(1, p->total_k / std::max(1, p->batch)) : p->seqlen_k;
+    const int64_t sh = a.shift_explicit ? a.shift_val : lk - lq;
+    auto keys_of = [&](int64_t i) {
+      const int64_t hi = a.wr >= 0 ? std::min(lk - 1, i + sh + a.wr) : lk - 1;
+      const int64_t lo = a.wl >= 0 ? std::max<int64_t>(0, i + sh - a.wl) : 0;
+      return std::max<int64_t>(0, hi - lo + 1) +
+             std::max<int64_t>(0, std::min<int64_t>(a.n_sink, std::min(lo, hi + 1)));
+    };
+    auto rows_of = [&](int64_t j) {
+      const int64_t i_lo = a.wr >= 0 ? std::max<int64_t>(0, j - sh - a.wr) : 0;
+      const int64_t i_hi = (a.wl >= 0 && j >= a.n_sink) ? std::min(lq - 1, j - sh + a.wl) : lq - 1;
+      return std::max<int64_t>(0, i_hi - i_lo + 1);
+    };
+    a.rev_q = keys_of(lq - 1) > keys_of(0);
+    a.rev_k = rows_of(lk - 1) > rows_of(0);
+  }
   a.scale = p->softmax_scale;
   a.scale_log2 = p->softmax_scale * kLog2e;
 

@@ -22,10 +22,13 @@
 //   S = Q K^T, dP = dO V^T      A = Q / dO row fragments (LDS), B = K (registers) / V (LDS)
 //   P = exp2(S*c - lse2), dS = P * (dP - delta)
 //   dV^T += dO^T P, dK^T += Q^T dS   A = transposing LDS reads of dO / Q, B = P / dS (regs)
-// Its MFMAs are inline assembly so that the register file of each accumulator can be
-// chosen: S and dP in vector registers (the vector ALU reads them next), dK^T and dV^T in
-// accumulation registers.  Left to the compiler, S and dP end up in accumulation registers
-// too and every element costs two copies.
+// The S and dP MFMAs are inline assembly so that their accumulators live in vector
+// registers, where the vector ALU reads them next; left to the compiler they end up in
+// accumulation registers like dK^T and dV^T and every element costs two copies.  The
+// compiler does not know that these statements are MFMAs and pads nothing after them:
+// the code keeps at least two later MFMAs between the last one that writes S or dP and
+// the first read of the result.  The dK^T / dV^T MFMAs are compiler builtins (accumulation
+// registers), so every copy or read the compiler adds around them is padded as required.
 // DQ per (key tile, wave); wave owns 32 query columns (C layout: lane = query):
 //   S^T = K Q^T, dP^T = V dO^T  A = K / V row fragments from LDS, B = Q / dO fragments (regs)
 //   dS^T as above with per-lane lse2 / delta
@@ -81,7 +84,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   const int u = lane >> 4;
 
   // ---- which (sequence, kv head, key tile) ---------------------------------
-  const int slot = wid % a.n_tile;
+  const int slot = a.rev_k ? a.n_tile - 1 - wid % a.n_tile : wid % a.n_tile;
   int rest = wid / a.n_tile;
   const int hk = rest % a.heads_kv;
   SeqInfo s;
@@ -381,12 +384,12 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
           if constexpr ((m - NG + 1) % GPC == 0) p_chunk(std::integral_constant<int, (m - NG + 1) / GPC - 1>{});
         } else if constexpr (m < 3 * NG) {
           constexpr int j = f - 2 * KS, ks2 = j / DB, d = j % DB;
-          M::mfma32_acc(fa[f], pb[kb][ks2], dv_acc[kb][d]);
+          dv_acc[kb][d] = M::mfma32(fa[f], pb[kb][ks2], dv_acc[kb][d]);
           if constexpr ((m - 2 * NG + 1) % GPC == 0)
             ds_chunk(std::integral_constant<int, (m - 2 * NG + 1) / GPC - 1>{});
         } else {
           constexpr int j = f - 3 * KS, ks2 = j / DB, d = j % DB;
-          M::mfma32_acc(fa[f], dsb[kb][ks2], dk_acc[kb][d]);
+          dk_acc[kb][d] = M::mfma32(fa[f], dsb[kb][ks2], dk_acc[kb][d]);
         }
         fence();
       });
@@ -401,9 +404,6 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   }
 
   // ---- write dK, dV (C layout: lane = key, regs = d) -----------------------------------
-  // (the MFMAs above are inline assembly: the compiler does not pad the distance between
-  // the last of them and the first read of their results)
-  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 #pragma unroll
   for (int kb = 0; kb < KB; kb++) {
     const int jc = jw0 + kb * 32 + l32;
@@ -469,7 +469,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(const AttnArgs a) {
   const int bm = pair ? 128 : 256;
   const int hu = wid % units;
   int rest = wid / units;
-  const int slot = rest % a.n_tile;
+  const int slot = a.rev_q ? a.n_tile - 1 - rest % a.n_tile : rest % a.n_tile;
   rest /= a.n_tile;
   const int hk = rest % a.heads_kv;
   const int hq = hk * a.group + (pair ? 2 * hu + (wave >> 2) : hu);

@@ -46,6 +46,10 @@ struct AttnArgs {
   int32_t dq_accumulate;  // backward: add to dq instead of overwriting it
   int32_t n_tile;          // tiles per sequence (dense) / total tile slots (packed)
   int32_t n_work;          // logical blocks
+  // Blocks are dispatched in logical order; these flags reverse the order of the query
+  // tiles (forward, dQ) or key tiles (dK/dV) so that the tiles with the most visible
+  // pairs start first and the short ones fill the tail of the launch.
+  int32_t rev_q, rev_k;
   float scale, scale_log2;
 };
 
@@ -117,17 +121,20 @@ struct Mma<__bf16> {
   static __device__ __forceinline__ f32x16 mfma32(V8 a, V8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
-  // The same instruction with the accumulator's register file chosen by the caller:
-  // accumulation registers (for accumulators only MFMAs touch) or vector registers (for
-  // accumulators the vector ALU reads next), and a zero-initialising form.
-  static __device__ __forceinline__ void mfma32_acc(V8 a, V8 b, f32x16& c) {
-    asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
-  }
+  // The same instruction as inline assembly with the accumulator kept in vector registers
+  // (for accumulators the vector ALU reads next; the builtin's accumulators live in
+  // accumulation registers), and a zero-initialising form (early clobber: the destination
+  // of a 32x32 MFMA must not overlap its A / B operands).  The compiler sees opaque
+  // statements and inserts no wait states after them: the caller keeps at least two later
+  // MFMAs (or 32 idle cycles) between one of these and any other instruction that reads
+  // its result, copies added by the register allocator included -- accumulators that live
+  // across control flow are therefore better served by the builtin.  Volatile: they keep
+  // their order among themselves and the empty volatile statements that pin vector work.
   static __device__ __forceinline__ void mfma32_vec(V8 a, V8 b, f32x16& c) {
-    asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
   }
   static __device__ __forceinline__ void mfma32_vec0(V8 a, V8 b, f32x16& c) {
-    asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=v"(c) : "v"(a), "v"(b));
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
   }
   static __device__ __forceinline__ V8 pack(const float* x) {
     f32x8 f = {x[0], x[1], x[2], x[3], x[4], x[5], x[6], x[7]};
@@ -146,14 +153,11 @@ struct Mma<_Float16> {
   static __device__ __forceinline__ f32x16 mfma32(V8 a, V8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
-  static __device__ __forceinline__ void mfma32_acc(V8 a, V8 b, f32x16& c) {
-    asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
-  }
   static __device__ __forceinline__ void mfma32_vec(V8 a, V8 b, f32x16& c) {
-    asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
   }
   static __device__ __forceinline__ void mfma32_vec0(V8 a, V8 b, f32x16& c) {
-    asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=v"(c) : "v"(a), "v"(b));
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
   }
   static __device__ __forceinline__ V8 pack(const float* x) {
     f32x8 f = {x[0], x[1], x[2], x[3], x[4], x[5], x[6], x[7]};

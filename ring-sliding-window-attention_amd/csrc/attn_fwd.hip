@@ -64,7 +64,7 @@ __global__ __launch_bounds__(512) void attn_fwd_kernel(const AttnArgs a) {
   const int bm = pair ? 128 : 256;                  // query rows per block
   const int hu = wid % units;
   int rest = wid / units;
-  const int slot = rest % a.n_tile;
+  const int slot = a.rev_q ? a.n_tile - 1 - rest % a.n_tile : rest % a.n_tile;
   rest /= a.n_tile;
   const int hk = rest % a.heads_kv;
   const int hq = hk * a.group + (pair ? 2 * hu + (wave >> 2) : hu);
