@@ -187,9 +187,15 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
     int64_t stat_row;  // index of row 0 of this head in the statistics arrays
   };
   const int i_first = qt_lo * C::BM;
+  // Every head's walk over the n_qt query tiles starts at tile qt_start and wraps around,
+  // chosen so that at any step all blocks of a kv head whose walks are equally long are
+  // on the same query tile modulo n_qt: neighbouring key tiles see almost the same query
+  // rows, and walking them in step lets one L2 fill serve all of them.
+  const int qt_start = n_qt > 0 ? (n_qt - qt_lo % n_qt) % n_qt : 0;
   Cursor nxt;  // the tile that the load parts fetch
-  nxt.qt = 0;
-  nxt.i0 = i_first;
+  nxt.qt = qt_start;
+  nxt.i0 = i_first + qt_start * C::BM;
+  int nxt_left = n_qt;  // tiles left in the walk of nxt's head, nxt included
   nxt.q_head = q_base + (int64_t)hk * a.group * a.q_st[2];
   nxt.do_head = do_base + (int64_t)hk * a.group * a.do_st[2];
   nxt.stat_row = (int64_t)hk * a.group * a.rows_q + ws_row0;
@@ -225,6 +231,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
     if (nxt.qt == n_qt) {
       nxt.qt = 0;
       nxt.i0 = i_first;
+    }
+    if (--nxt_left == 0) {
+      nxt_left = n_qt;
+      nxt.qt = qt_start;
+      nxt.i0 = i_first + qt_start * C::BM;
       nxt.q_head += a.q_st[2];
       nxt.do_head += a.do_st[2];
       nxt.stat_row += a.rows_q;
@@ -242,7 +253,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
 
   const char* v_lds = v_s + wave * (32 * KB) * C::ROWB;
 
-  int cur_i0 = i_first;  // first row of the tile being computed
+  int cur_i0 = i_first + qt_start * C::BM;  // first row of the tile being computed
   // For which first rows i0 of a 32-row tile does any (query, key of this wave) pair survive
   // the mask (need_*), and for which is no pair masked (full_*)?  With
   // i1 = min(i0 + 32, len_q) - 1 and the wave's keys jw0 .. jw1 the conditions
