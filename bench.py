@@ -253,6 +253,32 @@ def main():
                 "bwd_own_chunk_all_kernels": {"ms": bwd_med, "TFLOP/s": tf(10 * fl_pair, bwd_med),
                                               "flops_per_pair": "10 D (window-effective)"},
             }
+            # The dK/dV launch of the own-chunk block alone leaves a quarter of the compute
+            # units idle in its tail (256 blocks of unequal length on 256 units); in the rank
+            # step the previous-chunk dK/dV launch of the second stream fills them.  The
+            # pair, launched the way the step launches it, is timed here for reference.
+            pk, pv_ = prev.detach()[0][:, S - W:], prev.detach()[1][:, S - W:]
+            o_p, lse_p = o_d[:, :W], lse_d[:, :, :W]
+            dqp = torch.empty_like(qd[:, :W])
+            dkp, dvp = torch.empty_like(pk), torch.empty_like(pv_)
+            ws_p = torch.empty(W * HQ * 8 + 4096, dtype=torch.uint8, device=dev)
+            side = torch.cuda.Stream(dev)
+            attn_bwd(qd[:, :W], pk, pv_, o_p, lse_p, do[:, :W], dqp, dkp, dvp, None, (0, S), False,
+                     workspace=ws_p, phases=PREP)
+
+            def dkdv_pair():
+                side.wait_stream(torch.cuda.current_stream(dev))
+                with torch.cuda.stream(side):
+                    attn_bwd(qd[:, :W], pk, pv_, o_p, lse_p, do[:, :W], dqp, dkp, dvp, None,
+                             (0, S), False, workspace=ws_p, phases=DKDV)
+                bwd(DKDV)
+                torch.cuda.current_stream(dev).wait_stream(side)
+
+            pair_med, _ = event_ms(dkdv_pair, 20)
+            rec["kernels"]["bwd_dkdv_own_and_previous_chunk_concurrent"] = {
+                "ms": pair_med, "TFLOP/s": tf(8 * D * pairs * HQ, pair_med),
+                "pct_bf16_mfma_peak": 100.0 * tf(8 * D * pairs * HQ, pair_med) / PEAK_BF16_TFLOPS,
+                "flops_per_pair": "8 D", "note": "two launches on two streams, as in the rank step"}
             # config 2: plain single-GPU SWA, batch 2, seq 8192, 32/32 heads, window 1000
             q2, k2, v2, do2 = (mk(2, 8192, 32, 128) for _ in range(4))
             o2, l2 = attn_fwd(q2, k2, v2, None, (1000, 0), True)
