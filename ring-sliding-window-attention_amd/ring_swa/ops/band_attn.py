@@ -171,10 +171,12 @@ def attn_bwd(
     if softmax_scale is None:
         softmax_scale = q.shape[-1] ** (-0.5)
     if q.numel() == 0 or k.numel() == 0:
-        if not dq_accumulate:
+        # nothing to attend: the outputs of the requested phases are zero
+        if (phases & 4) and not dq_accumulate:
             dq.zero_()
-        dk.zero_()
-        dv.zero_()
+        if phases & 2:
+            dk.zero_()
+            dv.zero_()
         return
     p = _params(q, k, v, softmax_scale, window_size, causal, cu_seqlens_q, cu_seqlens_k, num_sink,
                 mask_shift)

@@ -254,3 +254,20 @@ def test_bwd_dq_accumulate_is_one_fp32_add_of_the_two_16bit_values(hq, hk, s):
     torch.cuda.synchronize()
     assert torch.equal(acc, (base.float() + dq.float()).bfloat16())
     assert torch.equal(dk2, dk) and torch.equal(dv2, dv)
+
+
+def test_bwd_empty_queries_write_only_the_outputs_of_the_requested_phases():
+    """No query rows: dK = dV = 0 and dQ is empty, but a call restricted to the dQ phase
+    must leave dK / dV (another call's results) alone."""
+    from ring_swa.ops import attn_bwd
+
+    q = torch.empty(1, 0, 4, 128, dtype=torch.bfloat16, device="cuda")
+    k = _rand((1, 96, 2, 128), torch.bfloat16, 2).cuda()
+    v = _rand((1, 96, 2, 128), torch.bfloat16, 3).cuda()
+    o, do, dq = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
+    lse = torch.empty(1, 4, 0, dtype=torch.float32, device="cuda")
+    dk, dv = torch.full_like(k, 7.0), torch.full_like(v, 7.0)
+    attn_bwd(q, k, v, o, lse, do, dq, dk, dv, None, (16, 0), True, phases=1 | 4)
+    assert bool((dk == 7).all()) and bool((dv == 7).all())
+    attn_bwd(q, k, v, o, lse, do, dq, dk, dv, None, (16, 0), True)
+    assert bool((dk == 0).all()) and bool((dv == 0).all())
