@@ -404,7 +404,7 @@ def ring_steps_varlen(cu_seqlens: Sequence[int], seq_len: int, window_size: int,
 
 
 # --------------------------------------------------------------------------
-# work counters (BASELINE FLOP model)
+# work counters (the FLOP model of the headline metric: 4 D per pair forward, 10 D backward)
 # --------------------------------------------------------------------------
 def band_pairs(length: int, window_size: int) -> int:
     """Unmasked (query,key) pairs of one sequence: closed form ``P(L,w)``."""
