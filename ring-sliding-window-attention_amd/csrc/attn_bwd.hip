@@ -2,7 +2,8 @@
 //
 // Replaces flash-attn's backward as wrapped at ring_swa/ops/wrap_flash.py:276-429.
 // Three launches on the caller's stream:
-//   PREP : per (row, q head): delta = sum_d dO * O and lse2 = lse * log2(e) (-inf -> +inf),
+//   PREP : per (row, q head): -delta = -sum_d dO * O and -lse2 = -lse * log2(e) (stored negated:
+//          they enter the kernels as addends),
 //          both fp32, into the caller's workspace
 //   DKDV : one block (4 waves, one per SIMD, up to 512 registers each) owns 256 keys of one
 //          (sequence, kv head) and walks the query tiles (32 rows) that can see them, for
@@ -20,7 +21,7 @@
 // DKDV per (query tile, wave) (C layout: lane = key; two 32-key blocks per wave, so every
 // fragment read from LDS feeds two MFMAs):
 //   S = Q K^T, dP = dO V^T      A = Q / dO row fragments (LDS), B = K (registers) / V (LDS)
-//   P = exp2(S*c - lse2), dS = P * (dP - delta)
+//   P = exp2(S*c - lse2), dS = P * (dP - delta); the dP chains start from -delta instead of zero
 //   dV^T += dO^T P, dK^T += Q^T dS   A = transposing LDS reads of dO / Q, B = P / dS (regs)
 // The S and dP MFMAs are inline assembly so that their accumulators live in vector
 // registers, where the vector ALU reads them next; left to the compiler they end up in
@@ -70,7 +71,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   __shared__ __attribute__((aligned(1024))) char q_s1[C::Q_TILE];
   __shared__ __attribute__((aligned(1024))) char do_s0[C::Q_TILE];
   __shared__ __attribute__((aligned(1024))) char do_s1[C::Q_TILE];
-  __shared__ __attribute__((aligned(1024))) float st_s0[2 * C::BM];  // lse2[BM], delta[BM]
+  __shared__ __attribute__((aligned(1024))) float st_s0[2 * C::BM];  // -lse2[BM], -delta[BM]
   __shared__ __attribute__((aligned(1024))) float st_s1[2 * C::BM];
 
   const int wid = logical_block_id(a.n_work);
@@ -292,7 +293,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
       // per MFMA, with scheduling fences between the groups.  Every fragment read from LDS
       // feeds the MFMAs of both key blocks; K comes from registers; fragments are fetched
       // AH fragment slots ahead; P = exp2(S c - lse2) is computed under the dP MFMAs and
-      // dS = P (dP - delta) under the dV MFMAs.
+      // dS = P (dP - delta) under the dV MFMAs; dP - delta comes out of the MFMAs, whose
+      // chains start from -delta in the accumulator layout.
       constexpr int NG = KB * KS;   // MFMAs per GEMM (KS = 2 DB)
       constexpr int NF = 4 * KS;    // fragment slots: Q, dO (+ V), dO^T, Q^T; KB MFMAs each
       constexpr int AH = 2;
@@ -321,7 +323,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
       const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f,
                            0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
       f32x16 sacc[KB], pacc[KB];
-      f32x4 l4[4], d4[4];
+      f32x16 dinit;  // -delta of the 32 rows in the accumulator layout: the dP chains start from it
+      f32x4 l4[4];   // -lse2 of the rows
       V8 pb[KB][2], dsb[KB][2];
       // vector work in 2 KB chunks of four rows: chunk order lets the packed operands of
       // the first k-step be complete first
@@ -338,8 +341,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
 #pragma unroll
         for (int e = 0; e < 4; e++) {
           const int i = 4 * i4 + e;
-          pk[kb][i] =
-              __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][i], a.scale_log2, -l4[i4][e]));
+          pk[kb][i] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][i], a.scale_log2, l4[i4][e]));
         }
         if (!full) {
           // key position relative to the aligned diagonal of row i0: rel(r) = rel0 - r
@@ -364,7 +366,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
 #pragma unroll
         for (int e = 0; e < 4; e++) {
           const int i = 4 * i4 + e;
-          dsk[kb][4 * (i4 & 1) + e] = pk[kb][i] * (pacc[kb][i] - d4[i4][e]);  // zero where P is
+          dsk[kb][4 * (i4 & 1) + e] = pk[kb][i] * pacc[kb][i];  // zero where P is
         }
         if (i4 & 1) dsb[kb][i4 >> 1] = M::pack(dsk[kb]);
       };
@@ -376,10 +378,13 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
         constexpr int f = m / KB, kb = m % KB;  // fragment slot and key block of this MFMA
         if constexpr (kb == 0) fetch(std::integral_constant<int, f + AH>{});
         if (m < NPART && has_next) load_part(m, qn, don, stn);
-        // row statistics: lse2 at the end of S, delta at the end of dP
+        // row statistics: -delta early in S (the dP chains start from it), -lse2 at its end
+        if constexpr (m >= 4 && m < 8) {
+          const f32x4 t4 = *(const f32x4*)(delta_lds + 8 * (m - 4) + 4 * g);
+#pragma unroll
+          for (int e = 0; e < 4; e++) dinit[4 * (m - 4) + e] = t4[e];
+        }
         if constexpr (m >= NG - 4 && m < NG) l4[m - (NG - 4)] = *(const f32x4*)(lse_lds + 8 * (m - (NG - 4)) + 4 * g);
-        if constexpr (m >= 2 * NG - 4 && m < 2 * NG)
-          d4[m - (2 * NG - 4)] = *(const f32x4*)(delta_lds + 8 * (m - (2 * NG - 4)) + 4 * g);
         if constexpr (m < NG) {
           if constexpr (f == 0) {
             M::mfma32_vec0(fa[f], kf[kb][f], sacc[kb]);
@@ -388,7 +393,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
           }
         } else if constexpr (m < 2 * NG) {
           if constexpr (f == KS) {
-            M::mfma32_vec0(fa[f], fv[kb][f - KS], pacc[kb]);
+            M::mfma32_vec_init(fa[f], fv[kb][f - KS], dinit, pacc[kb]);
           } else {
             M::mfma32_vec(fa[f], fv[kb][f - KS], pacc[kb]);
           }
@@ -529,7 +534,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(const AttnArgs a) {
 
   // Q / dO fragments (B operands): lane = query column, 8 consecutive d per k-step
   V8 qf[C::KSTEPS], dof[C::KSTEPS];
-  float lse2 = __builtin_inff(), delta = 0.f;
+  float lse2 = -__builtin_inff(), delta = 0.f;  // negated, as the workspace holds them
   if (iq < len_q) {
 #pragma unroll
     for (int ks = 0; ks < C::KSTEPS; ks++) {
@@ -611,8 +616,8 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(const AttnArgs a) {
         for (int t = 0; t < 2; t++)
 #pragma unroll
           for (int i = 0; i < 16; i++) {
-            const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[t][i], a.scale_log2, -lse2));
-            pacc[t][i] = p * (pacc[t][i] - delta);
+            const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[t][i], a.scale_log2, lse2));
+            pacc[t][i] = p * (pacc[t][i] + delta);
           }
       } else {
         const int hi_rel = rb.hi - j0;
@@ -624,8 +629,8 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(const AttnArgs a) {
           for (int i = 0; i < 16; i++) {
             const int j = t * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
             const bool ok = (j <= hi_rel) & ((j >= lo_rel) | (j < sink_rel));
-            const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[t][i], a.scale_log2, -lse2));
-            pacc[t][i] = ok ? p * (pacc[t][i] - delta) : 0.f;
+            const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[t][i], a.scale_log2, lse2));
+            pacc[t][i] = ok ? p * (pacc[t][i] + delta) : 0.f;
           }
       }
       // dQ^T[d, query] += K^T dS^T; dS^T is packed before the matrix section starts and the
@@ -705,8 +710,8 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(const AttnArgs a) {
 }
 
 // ============================================================================
-// row statistics: delta = sum_d dO * O and lse2 = lse * log2(e) (empty rows: +inf, so
-// that P = exp2(S*c - lse2) is zero).  One 16-lane (D=128) or 8-lane (D=64) group per
+// row statistics, stored negated: -delta = -sum_d dO * O and -lse2 = -lse * log2(e) (empty
+// rows: -inf, so that P = exp2(S*c - lse2) is zero).  One 16-lane (D=128) or 8-lane (D=64) group per
 // (row, head).
 // ============================================================================
 template <typename T, int D>
@@ -737,9 +742,9 @@ __global__ __launch_bounds__(256) void attn_bwd_prep_kernel(const AttnArgs a) {
 #pragma unroll
   for (int m = LPR / 2; m >= 1; m >>= 1) acc += __shfl_xor(acc, m, 64);
   if (c == 0) {
-    a.delta[(int64_t)h * a.rows_q + row] = acc;
+    a.delta[(int64_t)h * a.rows_q + row] = -acc;
     const float l = a.lse[l_off + h * a.lse_st[1]];
-    a.lse2[(int64_t)h * a.rows_q + row] = (l == -__builtin_inff()) ? __builtin_inff() : l * kLog2e;
+    a.lse2[(int64_t)h * a.rows_q + row] = (l == -__builtin_inff()) ? l : -l * kLog2e;
   }
 }
 

@@ -32,8 +32,8 @@ struct AttnArgs {
   void* dq;
   void* dk;
   void* dv;
-  float* delta;   // fp32 [heads_q, rows_q] packed: sum_d dO * O          (workspace)
-  float* lse2;    // fp32 [heads_q, rows_q] packed: lse * log2(e), -inf -> +inf (workspace)
+  float* delta;   // fp32 [heads_q, rows_q] packed: -sum_d dO * O         (workspace)
+  float* lse2;    // fp32 [heads_q, rows_q] packed: -lse * log2(e); empty rows -inf (workspace)
   const int32_t* cu_q;
   const int32_t* cu_k;
   int64_t q_st[3], k_st[3], v_st[3], o_st[3], do_st[3], dq_st[3], dk_st[3], dv_st[3], lse_st[3];
@@ -136,6 +136,10 @@ struct Mma<__bf16> {
   static __device__ __forceinline__ void mfma32_vec0(V8 a, V8 b, f32x16& c) {
     asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
   }
+  // first MFMA of a chain that starts from `init` instead of zero
+  static __device__ __forceinline__ void mfma32_vec_init(V8 a, V8 b, const f32x16& init, f32x16& c) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3" : "=&v"(c) : "v"(a), "v"(b), "v"(init));
+  }
   static __device__ __forceinline__ V8 pack(const float* x) {
     f32x8 f = {x[0], x[1], x[2], x[3], x[4], x[5], x[6], x[7]};
     return __builtin_convertvector(f, V8);
@@ -158,6 +162,10 @@ struct Mma<_Float16> {
   }
   static __device__ __forceinline__ void mfma32_vec0(V8 a, V8 b, f32x16& c) {
     asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
+  }
+  // first MFMA of a chain that starts from `init` instead of zero
+  static __device__ __forceinline__ void mfma32_vec_init(V8 a, V8 b, const f32x16& init, f32x16& c) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %3" : "=&v"(c) : "v"(a), "v"(b), "v"(init));
   }
   static __device__ __forceinline__ V8 pack(const float* x) {
     f32x8 f = {x[0], x[1], x[2], x[3], x[4], x[5], x[6], x[7]};
