@@ -21,6 +21,8 @@
  *                         ring_swa/sliding_window/varlen.py:406-417
  *   rswa_attn_bwd         ring_swa/ops/wrap_flash.py:276-327 (wrapped_flash_attn_bwd)
  *                         and :330-429 (wrapped_flash_attn_bwd_varlen)
+ *   rswa_attn_bwd_static  (no upstream counterpart: rswa_attn_bwd for callers that
+ *                         cannot allocate; see its declaration)
  *   rswa_attn_bwd_workspace_bytes   (sizing helper for the scratch rswa_attn_bwd
  *                         needs; upstream flash-attn allocates the same internally)
  */
@@ -177,6 +179,23 @@ int rswa_attn_bwd(const rswa_attn_params* p, void* stream);
 #define RSWA_BWD_DKDV 2
 #define RSWA_BWD_DQ 4
 int rswa_attn_bwd_phases(const rswa_attn_params* p, void* stream, int phases);
+
+/*
+ * rswa_attn_bwd without a caller workspace and without any allocation: the row statistics
+ * go to a buffer of RSWA_BWD_STATIC_MAX_BYTES that is part of the library's device image
+ * (every GPU the library runs on holds it until the process ends); p->workspace and
+ * p->workspace_bytes are ignored.  No counterpart in the upstream package: it is for
+ * callers that cannot allocate device memory around the call - code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  Shapes whose
+ * rswa_attn_bwd_workspace_bytes() exceed the buffer (more than 4 194 304 (row, q head)
+ * pairs) are refused with RSWA_ERR_UNSUPPORTED.  The buffer's address is looked up on the
+ * first call on each device (the device must be current, as for every other call); nothing
+ * in it has to be cleared between calls, the statistics kernel rewrites what the others
+ * read.  All calls on one GPU share the one buffer: calls that may overlap in time on the
+ * same GPU (different streams, different threads) race and must be serialised by the caller.
+ */
+#define RSWA_BWD_STATIC_MAX_BYTES (32u << 20)
+int rswa_attn_bwd_static(const rswa_attn_params* p, void* stream);
 
 /* Scratch rswa_attn_bwd needs for these shapes: two fp32 values per (row, q head) —
  * the row sum of dout * out and the LSE in base-2 units. */

@@ -40,6 +40,8 @@
 // that every access names its buffer statically (see attn_fwd.hip for why).
 #include "attn_common.h"
 
+#include <mutex>
+
 namespace rswa {
 namespace {
 
@@ -826,4 +828,63 @@ extern "C" int rswa_attn_bwd_phases(const rswa_attn_params* p, void* stream, int
 
 extern "C" int rswa_attn_bwd(const rswa_attn_params* p, void* stream) {
   return rswa_attn_bwd_phases(p, stream, RSWA_BWD_PREP | RSWA_BWD_DKDV | RSWA_BWD_DQ);
+}
+
+// ---- backward on the library's own statistics buffer --------------------------------------
+// The row statistics of rswa_attn_bwd_static live in this array instead of a caller
+// workspace.  In host code the array's name is only a handle: its device address is looked
+// up once per device (each GPU holds its own copy) and that pointer is what the kernels get.
+static __device__ __align__(256) unsigned char scratch[RSWA_BWD_STATIC_MAX_BYTES];
+
+namespace rswa {
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex scratch_mutex;
+void* scratch_ptr[kMaxDevices] = {nullptr};
+
+// Device address of `scratch` on the current device (nullptr + error message on failure).
+void* scratch_on_current_device() {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    fail(RSWA_ERR_LAUNCH, "attn_bwd_static: hipGetDevice: %s (device %d)", hipGetErrorString(e), dev);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(scratch_mutex);
+  if (!scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+      fail(RSWA_ERR_LAUNCH, "attn_bwd_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+      return nullptr;
+    }
+    scratch_ptr[dev] = ptr;
+  }
+  return scratch_ptr[dev];
+}
+}  // namespace
+}  // namespace rswa
+
+extern "C" int rswa_attn_bwd_static(const rswa_attn_params* p, void* stream) {
+  using namespace rswa;
+  RSWA_REQUIRE(p != nullptr, RSWA_ERR_INVALID, "attn_bwd_static: null params");
+  const uint64_t need = rswa_attn_bwd_workspace_bytes(p);
+  RSWA_REQUIRE(need <= RSWA_BWD_STATIC_MAX_BYTES, RSWA_ERR_UNSUPPORTED,
+               "attn_bwd_static: rows * heads_q needs %llu bytes of statistics, the built-in "
+               "buffer holds %llu (use rswa_attn_bwd with a caller workspace)",
+               (unsigned long long)need, (unsigned long long)RSWA_BWD_STATIC_MAX_BYTES);
+  rswa_attn_params q = *p;
+  // validate everything else before the device is touched (a placeholder keeps the
+  // workspace checks quiet; the real address replaces it below)
+  q.workspace = (void*)(uintptr_t)256;
+  q.workspace_bytes = RSWA_BWD_STATIC_MAX_BYTES;
+  {
+    AttnArgs probe;
+    int rc = fill_args(&q, true, probe);
+    if (rc != RSWA_OK) return rc;
+  }
+  void* ptr = scratch_on_current_device();
+  if (!ptr) return RSWA_ERR_LAUNCH;
+  q.workspace = ptr;
+  return rswa_attn_bwd(&q, stream);
 }

@@ -105,7 +105,7 @@ def lib() -> ctypes.CDLL:
         c_void_p, c_int, POINTER(c_int64),
         c_int64, c_int64, c_int64, c_int64, c_void_p,
     ]
-    for name in ("rswa_attn_fwd", "rswa_attn_bwd"):
+    for name in ("rswa_attn_fwd", "rswa_attn_bwd", "rswa_attn_bwd_static"):
         fn = getattr(L, name)
         fn.restype = c_int
         fn.argtypes = [POINTER(AttnParams), c_void_p]

@@ -144,6 +144,7 @@ def attn_bwd(
     workspace: Optional[torch.Tensor] = None,
     phases: int = 7,
     dq_accumulate: bool = False,
+    static_workspace: bool = False,
 ) -> None:
     """Masked attention backward; overwrites ``dq, dk, dv`` (views are fine).
 
@@ -151,7 +152,10 @@ def attn_bwd(
     per-call scratch allocation, and must be when the phases of one backward are spread
     over several calls; ``phases`` is the bit mask of ``rswa_attn_bwd_phases`` (1 prep,
     2 dk/dv kernel, 4 dq kernel).  ``dq_accumulate`` adds this call's dQ to the values
-    already in ``dq`` (fp32 add of the two 16-bit values, one rounding)."""
+    already in ``dq`` (fp32 add of the two 16-bit values, one rounding).
+    ``static_workspace=True`` runs the whole backward on the library's built-in statistics
+    buffer (``rswa_attn_bwd_static``): no device memory is allocated by the call; sizes
+    beyond the buffer raise ``NotImplementedError`` and overlapping calls on one GPU race."""
     packed = cu_seqlens_q is not None
     _check_qkv(q, k, v, packed)
     dev = _lib.require_device(q, k, v, o, softmax_lse, do, dq, dk, dv)
@@ -192,6 +196,11 @@ def attn_bwd(
     p.dk_stride = _lib.i64x3(_strides3(dk, packed))
     p.dv_stride = _lib.i64x3(_strides3(dv, packed))
     L = _lib.lib()
+    if static_workspace:
+        assert phases == 7 and workspace is None, "the built-in buffer serves whole backward calls"
+        with torch.cuda.device(dev):
+            _lib.check(L.rswa_attn_bwd_static(p, _lib.stream_ptr(dev)))
+        return
     need = int(L.rswa_attn_bwd_workspace_bytes(p))
     if workspace is None:
         workspace = torch.empty(need, dtype=torch.uint8, device=dev)  # 512-B aligned by torch

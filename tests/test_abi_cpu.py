@@ -82,3 +82,18 @@ def test_ops_refuse_cpu_tensors():
     l = torch.zeros(1, 2, 8)
     with pytest.raises(RuntimeError, match="no CPU path"):
         merge_attn_out(o, l, o.clone(), l.clone())
+
+
+def test_static_backward_refuses_oversize_without_a_gpu():
+    _ensure_built()
+    from ring_swa import _lib
+
+    L = _lib.lib()
+    p = _lib.AttnParams()
+    p.dtype, p.head_dim, p.batch, p.heads_q, p.heads_kv = 0, 128, 1, 32, 8
+    p.seqlen_q, p.seqlen_k = 131073, 8  # one row more than the built-in buffer serves
+    p.softmax_scale = 1.0
+    assert L.rswa_attn_bwd_workspace_bytes(p) > (32 << 20)
+    rc = L.rswa_attn_bwd_static(p, None)
+    assert rc == -2 and b"built-in" in L.rswa_last_error()
+    assert L.rswa_attn_bwd_static(None, None) == -1

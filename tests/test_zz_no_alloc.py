@@ -1,0 +1,73 @@
+"""The allocation-free backward entry point (``rswa_attn_bwd_static``, statistics in the
+library's own device buffer) gives bit for bit what ``rswa_attn_bwd`` gives with a caller
+workspace: same kernels, same order.  Two calls in a row, the second on a smaller input, so
+that stale statistics of the first call would show; then a size beyond the buffer is refused.
+Collected last on purpose (file name): a failure here must not hide the other tests."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(seed, b, s, hq, hk, d, window, packed_cu=None):
+    g = torch.Generator().manual_seed(seed)
+    if packed_cu is None:
+        shape_q, shape_k = (b, s, hq, d), (b, s, hk, d)
+    else:
+        shape_q, shape_k = (s, hq, d), (s, hk, d)
+    q, do = (torch.randn(*shape_q, generator=g).bfloat16().cuda() for _ in range(2))
+    k, v = (torch.randn(*shape_k, generator=g).bfloat16().cuda() for _ in range(2))
+    return q, k, v, do
+
+
+def _both(q, k, v, do, window, cu=None):
+    from ring_swa.ops import attn_bwd, attn_fwd
+
+    out, lse = attn_fwd(q, k, v, None, window, True, cu, cu)
+    grads = []
+    for static in (False, True):
+        dq, dk, dv = (torch.full_like(t, float("nan")) for t in (q, k, v))
+        before = torch.cuda.memory_allocated()
+        attn_bwd(q, k, v, out, lse, do, dq, dk, dv, None, window, True, cu, cu,
+                 static_workspace=static)
+        if static:
+            assert torch.cuda.memory_allocated() == before, "the static entry point allocated"
+        grads.append((dq, dk, dv))
+    torch.cuda.synchronize()
+    return grads
+
+
+def test_static_backward_equals_workspace_backward_twice_in_a_row():
+    # first call: 2 x 1536 rows x 8 heads; second, smaller: packed 700 rows x 4 heads
+    q, k, v, do = _case(0, 2, 1536, 8, 2, 128, (200, 0))
+    (a, b) = _both(q, k, v, do, (200, 0))
+    for x, y in zip(a, b):
+        assert not torch.isnan(y.float()).any()
+        assert torch.equal(x, y)
+    cu = torch.tensor([0, 130, 131, 500, 700], dtype=torch.int32, device="cuda")
+    q, k, v, do = _case(1, 1, 700, 4, 4, 64, (64, 0), packed_cu=cu)
+    (a, b) = _both(q, k, v, do, (64, 0), cu)
+    for x, y in zip(a, b):
+        assert not torch.isnan(y.float()).any()
+        assert torch.equal(x, y)
+
+
+def test_static_backward_refuses_sizes_beyond_its_buffer():
+    from ring_swa import _lib
+    from ring_swa.ops import band_attn
+
+    # 4 194 304 + 32 (row, head) pairs: one head row more than the buffer holds
+    rows, heads = 131073, 32
+    q = torch.empty(1, 8, heads, 128, dtype=torch.bfloat16, device="cuda")
+    p = band_attn._params(q, q, q, 1.0, (8, 0), True, None, None, 0)
+    p.seqlen_q = rows
+    p.seqlen_k = 8
+    for name in ("out", "lse", "dout", "dq", "dk", "dv"):
+        setattr(p, name, q.data_ptr())
+    st = _lib.i64x3((rows * heads * 128, heads * 128, 128))
+    for name in ("out_stride", "dout_stride", "dq_stride", "dk_stride", "dv_stride"):
+        setattr(p, name, st)
+    p.lse_stride = _lib.i64x3((heads * rows, rows, 1))
+    rc = _lib.lib().rswa_attn_bwd_static(p, None)
+    assert rc == -2
+    assert b"built-in" in _lib.lib().rswa_last_error()
