@@ -8,6 +8,7 @@ from __future__ import annotations
 
 import concurrent.futures as cf
 import os
+import re
 import shutil
 import subprocess
 import sys
@@ -31,6 +32,8 @@ FLAGS = [
     "-Wno-unknown-attributes",
     # packed fp32 VALU forms are kept out of generated code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # per-kernel register / scratch report on stderr (checked below)
+    "-Rpass-analysis=kernel-resource-usage",
 ]
 
 
@@ -65,11 +68,45 @@ def _compile(src: str, force: bool) -> str:
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError(f"hipcc failed for {src}:\n{r.stdout}\n{r.stderr}")
-        noise = "packed-fp32-ops"
-        warn = "\n".join(l for l in r.stderr.splitlines() if noise not in l and l.strip())
+        _check_no_scratch(src, r.stderr)
+        warn = _real_warnings(r.stderr)
         if warn:
             sys.stderr.write(warn + "\n")
     return obj
+
+
+def _real_warnings(stderr: str) -> str:
+    """Compiler output minus the resource-usage remarks (each followed by a source line and
+    a caret line) and the host pass's note about the device-only target feature."""
+    out, skip = [], 0
+    for line in stderr.splitlines():
+        if skip:
+            skip -= 1
+            continue
+        if "-Rpass-analysis=kernel-resource-usage" in line:
+            skip = 2 if "Function Name" in line else 0
+            continue
+        if "packed-fp32-ops" in line or not line.strip():
+            continue
+        out.append(line)
+    return "\n".join(out)
+
+
+def _check_no_scratch(src: str, stderr: str) -> None:
+    """No kernel may use scratch memory: a register spilled inside a tile loop comes back
+    through a load whose wait also waits for every tile load in flight."""
+    name, bad = None, []
+    for line in stderr.splitlines():
+        m = re.search(r"remark:\s+(.*?): (.*?) \[-Rpass-analysis=kernel-resource-usage\]", line)
+        if not m:
+            continue
+        key, val = m.group(1).strip(), m.group(2).strip()
+        if key == "Function Name":
+            name = val
+        elif key.startswith("ScratchSize") and val != "0":
+            bad.append(f"{name}: {val} bytes of scratch per lane")
+    if bad:
+        raise RuntimeError(f"{src}: kernels spill registers to scratch memory:\n  " + "\n  ".join(bad))
 
 
 def build(force: bool = False, jobs: int = 8) -> str:

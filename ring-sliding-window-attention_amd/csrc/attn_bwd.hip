@@ -322,8 +322,6 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
           fa[f] = tr_pair<V8>(src + off0, src + off1);
         }
       };
-      const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f,
-                           0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
       f32x16 sacc[KB], pacc[KB];
       f32x16 dinit;  // -delta of the 32 rows in the accumulator layout: the dP chains start from it
       f32x4 l4[4];   // -lse2 of the rows
@@ -422,9 +420,14 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   }
 
   // ---- write dK, dV (C layout: lane = key, regs = d) -----------------------------------
+  // The lane's position is taken afresh (opaque to the optimiser): addresses derived from
+  // values computed before the walk would be kept in registers across it, and spilled.
+  int lane_e = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+  asm volatile("" : "+v"(lane_e));
+  const int l32_e = lane_e & 31, g_e = lane_e >> 5;
 #pragma unroll
   for (int kb = 0; kb < KB; kb++) {
-    const int jc = jw0 + kb * 32 + l32;
+    const int jc = jw0 + kb * 32 + l32_e;
     if (jc < len_k) {
 #pragma unroll
       for (int mtx = 0; mtx < 2; mtx++) {  // 0: dK, 1: dV
@@ -437,7 +440,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
             const f32x16& acc = mtx == 0 ? dk_acc[kb][d] : dv_acc[kb][d];
             const auto h4 = M::pack4(acc[4 * i4] * sc, acc[4 * i4 + 1] * sc, acc[4 * i4 + 2] * sc,
                                      acc[4 * i4 + 3] * sc);
-            *(typename M::V4*)(dst + d * 32 + 8 * i4 + 4 * g) = h4;
+            *(typename M::V4*)(dst + d * 32 + 8 * i4 + 4 * g_e) = h4;
           }
       }
     }
@@ -528,7 +531,6 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(const AttnArgs a) {
 
   const int r0 = i0 + (pair ? wave & 3 : wave) * 32;
   const int iq = r0 + l32;
-  const RowBounds rb = row_bounds(a, iq, len_q, len_k);
   const bool wave_valid = r0 < len_q;
   const bool wave_rows_full = r0 + 31 < len_q;
   const RowBounds wb_first = row_bounds(a, r0, len_q, len_k);
@@ -622,6 +624,12 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(const AttnArgs a) {
             pacc[t][i] = p * (pacc[t][i] + delta);
           }
       } else {
+        // edge tile: the lane's own mask bounds are recomputed here (only a few tiles per
+        // block take this path; kept across the loop they cost two registers, i.e. spills)
+        int lane_m = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+        asm volatile("" : "+v"(lane_m));
+        const RowBounds rb = row_bounds(a, r0 + (lane_m & 31), len_q, len_k);
+        const int g_m = lane_m >> 5;
         const int hi_rel = rb.hi - j0;
         const int lo_rel = rb.lo - j0;
         const int sink_rel = a.n_sink - j0;
@@ -629,7 +637,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(const AttnArgs a) {
         for (int t = 0; t < 2; t++)
 #pragma unroll
           for (int i = 0; i < 16; i++) {
-            const int j = t * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
+            const int j = t * 32 + 8 * (i >> 2) + 4 * g_m + (i & 3);
             const bool ok = (j <= hi_rel) & ((j >= lo_rel) | (j < sink_rel));
             const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[t][i], a.scale_log2, lse2));
             pacc[t][i] = ok ? p * (pacc[t][i] + delta) : 0.f;
@@ -735,6 +743,16 @@ __global__ __launch_bounds__(256) void attn_bwd_prep_kernel(const AttnArgs a) {
     do_off = bb * a.do_st[0] + i * a.do_st[1];
     l_off = bb * a.lse_st[0] + i * a.lse_st[2];
   }
+  // Packed rows past the last sequence belong to nobody: their out / dout may hold anything
+  // (NaN included), and the tile kernels read the statistics of the rows that follow a
+  // sequence's last tile.  They get the neutral pair, which keeps P and dS exactly zero.
+  if (a.cu_q && row >= a.cu_q[a.batch]) {
+    if (c == 0) {
+      a.delta[(int64_t)h * a.rows_q + row] = 0.f;
+      a.lse2[(int64_t)h * a.rows_q + row] = -__builtin_inff();
+    }
+    return;
+  }
   using V8 = typename Mma<T>::V8;
   const V8 o8 = *(const V8*)((const T*)a.out + o_off + h * a.o_st[2] + c);
   const V8 d8 = *(const V8*)((const T*)a.dout + do_off + h * a.do_st[2] + c);
@@ -767,6 +785,7 @@ int launch_bwd(AttnArgs& a, hipStream_t stream, int phases) {
   const int64_t units = a.rows_q * a.heads_q;
   if (units > 0 && (phases & RSWA_BWD_PREP)) {
     const unsigned blocks = (unsigned)ceil_div(units * (D / 8), 256);
+    clear_launch_error();
     hipLaunchKernelGGL((attn_bwd_prep_kernel<T, D>), dim3(blocks), dim3(256), 0, stream, a);
     int rc = check_launch("attn_bwd prep");
     if (rc != RSWA_OK) return rc;
@@ -781,6 +800,7 @@ int launch_bwd(AttnArgs& a, hipStream_t stream, int phases) {
       a.n_work = a.n_tile * a.heads_kv * a.batch;
     }
     if (a.n_work > 0) {
+      clear_launch_error();
       hipLaunchKernelGGL((attn_bwd_dkdv_kernel<T, D>), dim3(padded_grid(a.n_work)),
                          dim3(C::THREADS), 0, stream, a);
       int rc = check_launch("attn_bwd dkdv");
@@ -800,6 +820,7 @@ int launch_bwd(AttnArgs& a, hipStream_t stream, int phases) {
       a.n_work = a.n_tile * units_q * a.batch;
     }
     if (a.n_work > 0) {
+      clear_launch_error();
       hipLaunchKernelGGL((attn_bwd_dq_kernel<T, D>), dim3(padded_grid(a.n_work)),
                          dim3(C::THREADS), 0, stream, a);
       int rc = check_launch("attn_bwd dq");

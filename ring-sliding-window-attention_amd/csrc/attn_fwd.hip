@@ -368,6 +368,7 @@ int launch_fwd(AttnArgs& a, hipStream_t stream) {
     a.n_work = a.n_tile * units * a.batch;
   }
   if (a.n_work == 0) return RSWA_OK;
+  clear_launch_error();
   hipLaunchKernelGGL((attn_fwd_kernel<T, D>), dim3(padded_grid(a.n_work)), dim3(C::THREADS), 0,
                      stream, a);
   return check_launch("attn_fwd");

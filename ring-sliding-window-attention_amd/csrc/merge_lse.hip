@@ -165,6 +165,7 @@ int launch_merge(const MergeArgs& a, int64_t batch, hipStream_t stream) {
     args.n_stile = (int)ceil_div(a.seqlen, BS);
     const int64_t blocks = (int64_t)args.n_stile * a.heads * batch;
     if (blocks == 0) return;
+    clear_launch_error();
     hipLaunchKernelGGL((merge_kernel<TO, TN, LPR>), dim3((unsigned)blocks), dim3(kThreads), 0,
                        stream, args);
   };

@@ -19,6 +19,9 @@ int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
     if (!(cond)) return ::rswa::fail((code), __VA_ARGS__); \
   } while (0)
 
+// A launch is bracketed by these two: the first drops whatever error an earlier, unrelated
+// HIP call of this thread left behind, so that the second reports the launch's own only.
+inline void clear_launch_error() { (void)hipGetLastError(); }
 inline int check_launch(const char* what) {
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(RSWA_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));

@@ -120,6 +120,11 @@ def attn_fwd(
         lse = torch.empty((q.shape[0], q.shape[2], q.shape[1]), dtype=torch.float32, device=dev)
     if q.numel() == 0:
         return out, lse
+    if k.numel() == 0:
+        # no keys at all: every row is empty (out = 0, lse = -inf), as attn_bwd assumes
+        out.zero_()
+        lse.fill_(float("-inf"))
+        return out, lse
     p = _params(q, k, v, softmax_scale, window_size, causal, cu_seqlens_q, cu_seqlens_k, num_sink,
                 mask_shift)
     p.out = out.data_ptr()

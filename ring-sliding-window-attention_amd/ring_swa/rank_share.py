@@ -15,6 +15,7 @@ KV + dKV backward around the ring.
 from __future__ import annotations
 
 import math
+import threading
 from typing import List, Optional, Sequence, Tuple
 
 import torch
@@ -162,15 +163,19 @@ _SIDE_STREAMS = {}
 
 
 def _fork(device: torch.device) -> "torch.cuda.Stream":
-    """Side stream (default priority, one per device) ordered after the current stream.
+    """Side stream (default priority, one per device and host thread) ordered after the
+    current stream.
 
     The blocks of one step are independent until they are merged, and each launch alone
     leaves compute units idle in its tail (few, unequal work groups), so the diagonal
     block runs on the caller's stream and the other blocks on this one; ``_join``
-    orders the caller's stream after them again."""
-    side = _SIDE_STREAMS.get(device.index)
+    orders the caller's stream after them again.  Tensors used on the side stream are
+    allocated on the caller's stream before the fork (or marked with ``record_stream``), so
+    the caching allocator hands their memory back to the caller's stream only."""
+    key = (device.index, threading.get_ident())
+    side = _SIDE_STREAMS.get(key)
     if side is None:
-        side = _SIDE_STREAMS[device.index] = torch.cuda.Stream(device)
+        side = _SIDE_STREAMS[key] = torch.cuda.Stream(device)
     side.wait_stream(torch.cuda.current_stream(device))
     return side
 
@@ -183,6 +188,7 @@ def _forward_blocks(q, k, v, prev_kv, plan, scale, local_cu, ring_dtypes):
     """Run the planned blocks and merge them.  Dense 4-d tensors (batch 1 when packed)."""
     assert plan and plan[0][0] == 0, "the diagonal block comes first: it covers every row"
     side = _fork(q.device) if len(plan) > 1 else None
+    caller = torch.cuda.current_stream(q.device)
     parts = []
     for (i, qs, ks, window, causal) in plan:
         if i == 0:
@@ -195,12 +201,18 @@ def _forward_blocks(q, k, v, prev_kv, plan, scale, local_cu, ring_dtypes):
             kk, vv = prev_kv[i - 1][0], prev_kv[i - 1][1]
             with torch.cuda.stream(side):
                 o_i, l_i = attn_fwd(q[:, qs], kk[:, ks], vv[:, ks], scale, window, causal)
+            # allocated under the side stream, read by the merge on the caller's stream
+            o_i.record_stream(caller)
+            l_i.record_stream(caller)
         parts.append((qs, o_i, l_i))
     if side is not None:
         _join(side, q.device)
     _, out, lse = parts[0]
-    if ring_dtypes:
-        # accumulator types of ring_swa/sliding_window/nonvarlen.py:53-59
+    if ring_dtypes or len(parts) > 2:
+        # accumulator types of ring_swa/sliding_window/nonvarlen.py:53-59.  With two blocks
+        # the 16-bit running output is merged once and rounded once, the same bits as the
+        # fp32 accumulator gives; from three blocks on every further merge would add a
+        # rounding the reference does not have, so the fp32 / fp64 pair is used regardless.
         out, lse = out.float(), lse.double()
     for qs, o_i, l_i in parts[1:]:
         merge_attn_out(out[:, qs], lse[:, :, qs], o_i, l_i)

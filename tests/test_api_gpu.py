@@ -11,18 +11,14 @@ from oracle import attention_oracle as O
 
 pytestmark = pytest.mark.gpu
 
-OUT_TOL, GRAD_TOL = 2e-2, 5e-2
+from gradcheck_util import GRAD_TOL, relnorm as _relnorm  # noqa: E402
+
+OUT_TOL = 2e-2
 
 
 def _rand(shape, seed, dtype=torch.bfloat16):
     g = torch.Generator().manual_seed(seed)
     return torch.randn(*shape, generator=g).to(dtype)
-
-
-def _relnorm(x, ref):
-    x = x.float().cpu()
-    assert not torch.isnan(x).any()
-    return (x - ref).norm().item() / max(ref.norm().item(), 1e-30)
 
 
 def _gpu_fwd_bwd(fn, q, k, v, do):

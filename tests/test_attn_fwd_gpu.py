@@ -172,3 +172,19 @@ def test_fwd_rejects_bad_arguments():
         wrapped_flash_attn_fwd(qf, qf, qf, None, (1, 0), True)        # fp32
     with pytest.raises(ValueError):
         wrapped_flash_attn_fwd(q, q, q, -1.0, (1, 0), True)           # scale <= 0
+
+
+def test_fwd_without_any_key_gives_the_empty_row_pair():
+    """An empty KV slice: every row is empty, out = 0 and lse = -inf (the merge identity),
+    the same convention the backward assumes for it."""
+    from ring_swa.ops import attn_bwd, attn_fwd
+
+    q = torch.randn(2, 37, 4, 128, device="cuda").bfloat16()
+    k = torch.empty(2, 0, 2, 128, device="cuda", dtype=torch.bfloat16)
+    out, lse = attn_fwd(q, k, k.clone(), None, (16, 0), True)
+    assert out.shape == q.shape and (out == 0).all()
+    assert lse.shape == (2, 4, 37) and torch.isinf(lse).all() and (lse < 0).all()
+    dq, dk, dv = torch.full_like(q, 3.0), torch.empty_like(k), torch.empty_like(k)
+    attn_bwd(q, k, k.clone(), out, lse, torch.ones_like(q), dq, dk, dv, None, (16, 0), True)
+    torch.cuda.synchronize()
+    assert (dq == 0).all()

@@ -5,7 +5,7 @@ forward and backward.  One GQA group -- kv head 0 with the q heads that share it
 dK / dV depend on no other head -- is then checked against the oracle's masked softmax
 evaluated in fp32 on the same inputs (on the GPU: at these sizes the oracle's score
 matrices take seconds there and hours on host cores).  Tolerances are those of the path:
-out max-abs 2e-2, LSE 1e-3, dQ / dK / dV relative norm 5e-2.  Every other head is covered
+out max-abs 2e-2, LSE 1e-3, dQ / dK / dV relative norm 5e-2 (held to 1e-2 here).  Every other head is covered
 by properties that need no reference: finite values, and run-to-run bit equality of the
 (atomic-free) kernels.
 """
@@ -19,7 +19,7 @@ from oracle import attention_oracle as O
 
 pytestmark = pytest.mark.gpu
 
-OUT_TOL, LSE_TOL, GRAD_TOL = 2e-2, 1e-3, 5e-2
+OUT_TOL, LSE_TOL, GRAD_TOL = 2e-2, 1e-3, 1e-2
 D = 128
 
 

@@ -321,3 +321,41 @@ def test_pair_counters_match_masks():
     assert O.band_pairs(8192, 1000) == 7_699_692
     assert O.band_pairs(1024, 256) == 230_272
     assert O.band_pairs(8192, 4096) + 4096 * 4097 // 2 == 33_562_624 == 8192 * 4097
+
+
+def test_flop_counter_reproduces_the_quoted_workloads():
+    """4 / 10 / 14 x D x pairs x heads x batch against the totals quoted for the benchmark
+    shapes (0.2523 / 0.6308 / 0.8831 TFLOP for batch 2, 8192 tokens, 32 heads, window 1000;
+    0.5499 / 1.3747 / 1.9246 TFLOP for the rank share; 0.83 GFLOP for the CPU case) and
+    against a direct count on a small mask."""
+    f, b, t = O.attention_flops(O.band_pairs(8192, 1000), 128, 32, 2)
+    assert (round(f / 1e12, 4), round(b / 1e12, 4), round(t / 1e12, 4)) == (0.2523, 0.6308, 0.8831)
+    f, b, t = O.attention_flops(8192 * 4097, 128, 32)
+    assert (round(f / 1e12, 4), round(b / 1e12, 4), round(t / 1e12, 4)) == (0.5499, 1.3747, 1.9246)
+    assert round(O.attention_flops(O.band_pairs(1024, 256), 64, 4)[2] / 1e9, 2) == 0.83
+    m = O.window_allowed(9, 9, (3, 0), True)
+    # one multiply-add per (pair, d) and GEMM: forward 2 GEMMs, backward 5
+    assert O.attention_flops(int(m.sum()), 16, 3, 2) == tuple(
+        g * 2 * int(m.sum()) * 16 * 3 * 2 for g in (2, 5, 7))
+
+
+def test_global_mask_with_sinks_equals_the_per_sequence_rule():
+    """The sink branch of the global formula: per sequence it is the dense rule with sinks
+    (pinned above by brute force), and no pair ever crosses a sequence boundary."""
+    cu = [0, 5, 6, 17, 30]
+    total = cu[-1]
+    pos = torch.arange(total)
+    sid = torch.bucketize(pos, torch.tensor(cu[1:]), right=True)
+    start = torch.tensor(cu)[sid]
+    for w in (0, 2, 7, 40):
+        for n in (1, 4):
+            got = O.global_band_allowed(pos, pos, sid, sid, w, n_sink=n, seq_start_k=start)
+            want = torch.zeros(total, total, dtype=torch.bool)
+            for a, b in zip(cu[:-1], cu[1:]):
+                want[a:b, a:b] = O.window_allowed(b - a, b - a, (w, 0), True, n_sink=n)
+            assert torch.equal(got, want), (w, n)
+            # brute force of the stated rule
+            for p in range(total):
+                for t in range(total):
+                    rule = sid[p] == sid[t] and t <= p and (p - t <= w or t - cu[sid[t]] < n)
+                    assert bool(got[p, t]) == bool(rule)
