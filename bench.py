@@ -130,6 +130,7 @@ def main():
 
     import ring_swa
     from ring_swa.ops import attn_bwd, attn_fwd, merge_attn_out
+    from ring_swa.ops.band_attn import bwd_workspace_bytes
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
@@ -216,7 +217,7 @@ def main():
         qd, kd, vd = q.detach(), k.detach(), v.detach()
         o_d, lse_d = attn_fwd(qd, kd, vd, None, (W, 0), True)
         dq, dk, dv = torch.empty_like(qd), torch.empty_like(kd), torch.empty_like(vd)
-        ws = torch.empty(S * HQ * 8 + 4096, dtype=torch.uint8, device=dev)
+        ws = torch.empty(bwd_workspace_bytes(qd, kd), dtype=torch.uint8, device=dev)
         bwd = lambda ph: attn_bwd(qd, kd, vd, o_d, lse_d, do, dq, dk, dv, None, (W, 0), True,  # noqa: E731
                                   workspace=ws, phases=ph)
         bwd(7)
@@ -261,7 +262,7 @@ def main():
             o_p, lse_p = o_d[:, :W], lse_d[:, :, :W]
             dqp = torch.empty_like(qd[:, :W])
             dkp, dvp = torch.empty_like(pk), torch.empty_like(pv_)
-            ws_p = torch.empty(W * HQ * 8 + 4096, dtype=torch.uint8, device=dev)
+            ws_p = torch.empty(bwd_workspace_bytes(qd[:, :W], pk), dtype=torch.uint8, device=dev)
             side = torch.cuda.Stream(dev)
             attn_bwd(qd[:, :W], pk, pv_, o_p, lse_p, do[:, :W], dqp, dkp, dvp, None, (0, S), False,
                      workspace=ws_p, phases=PREP)

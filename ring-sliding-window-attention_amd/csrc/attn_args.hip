@@ -12,10 +12,38 @@ static uint64_t delta_bytes(const rswa_attn_params* p) {
   return align_up(rows * (uint64_t)p->heads_q * sizeof(float), 256);
 }
 
-uint64_t bwd_workspace_bytes(const rswa_attn_params* p) {
-  if (!p || p->batch <= 0 || p->heads_q <= 0 || p->head_dim <= 0) return 0;
-  return 2 * delta_bytes(p);
+BwdLayout bwd_layout(const rswa_attn_params* p, bool allow_split) {
+  BwdLayout L{};
+  L.nsplit = 1;
+  if (!p || p->batch <= 0 || p->heads_q <= 0 || p->heads_kv <= 0 || p->head_dim <= 0) return L;
+  L.stats_bytes = delta_bytes(p);
+  const bool packed = p->cu_seqlens_q != nullptr;
+  const int64_t rows_k = packed ? p->total_k : p->seqlen_k;
+  L.n_tile_k = (int)((rows_k + kDkvKeysPerBlock - 1) / kDkvKeysPerBlock + (packed ? p->batch : 0));
+  const int64_t blocks = (int64_t)L.n_tile_k * p->heads_kv * (packed ? 1 : p->batch);
+  const int group = p->heads_q / p->heads_kv;
+  // Splitting pays when one block per key tile leaves compute units without any work (see
+  // kDkvSplitBelow).  The parts of a tile are summed in a fixed order.
+  if (allow_split && group > 1 && blocks > 0 && blocks < kDkvSplitBelow) {
+    for (int n : {4, 3, 2})
+      if (group % n == 0) {
+        L.nsplit = n;
+        break;
+      }
+  }
+  L.count_off = 2 * L.stats_bytes;
+  L.part_off = L.count_off;
+  L.total_bytes = 2 * L.stats_bytes;
+  if (L.nsplit > 1) {
+    L.n_count = (int)blocks;
+    L.part_off = L.count_off + align_up((uint64_t)blocks * sizeof(int32_t), 256);
+    const uint64_t per_unit = (uint64_t)kDkvKeysPerBlock * p->head_dim * 2 * sizeof(float);
+    L.total_bytes = L.part_off + (uint64_t)blocks * L.nsplit * per_unit;
+  }
+  return L;
 }
+
+uint64_t bwd_workspace_bytes(const rswa_attn_params* p) { return bwd_layout(p, true).total_bytes; }
 
 static bool rows_aligned(const void* ptr, const int64_t* st) {
   if (((uintptr_t)ptr) % 16) return false;
@@ -24,7 +52,7 @@ static bool rows_aligned(const void* ptr, const int64_t* st) {
   return true;
 }
 
-int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a) {
+int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a, bool allow_split) {
   RSWA_REQUIRE(p != nullptr, RSWA_ERR_INVALID, "attn: null params");
   RSWA_REQUIRE(p->dtype == RSWA_BF16 || p->dtype == RSWA_F16, RSWA_ERR_UNSUPPORTED,
                "attn: dtype %d (only bf16 and fp16)", p->dtype);
@@ -73,6 +101,10 @@ int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a) {
   a.dv = p->dv;
   a.delta = nullptr;
   a.lse2 = nullptr;
+  a.dkv_part = nullptr;
+  a.dkv_count = nullptr;
+  a.nsplit = 1;
+  a.n_count = 0;
   a.cu_q = p->cu_seqlens_q;
   a.cu_k = p->cu_seqlens_k;
   for (int i = 0; i < 3; i++) {
@@ -140,7 +172,8 @@ int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a) {
       RSWA_REQUIRE(rq * p->dout_stride[1] * 2 < (1ll << 31) - 65536 && p->dout_stride[1] >= 0,
                    RSWA_ERR_UNSUPPORTED, "attn_bwd: one sequence of dout spans 2 GiB or more");
     }
-    const uint64_t need = bwd_workspace_bytes(p);
+    const BwdLayout L = bwd_layout(p, allow_split);
+    const uint64_t need = L.total_bytes;
     RSWA_REQUIRE(p->workspace != nullptr || need == 0, RSWA_ERR_INVALID,
                  "attn_bwd: null workspace");
     RSWA_REQUIRE(p->workspace_bytes >= need, RSWA_ERR_INVALID,
@@ -150,6 +183,10 @@ int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a) {
                  "attn_bwd: workspace must be 256-byte aligned");
     a.lse2 = (float*)p->workspace;
     a.delta = (float*)((char*)p->workspace + delta_bytes(p));
+    a.nsplit = L.nsplit;
+    a.n_count = L.n_count;
+    a.dkv_count = (int32_t*)((char*)p->workspace + L.count_off);
+    a.dkv_part = (float*)((char*)p->workspace + L.part_off);
     RSWA_REQUIRE(2 * delta_bytes(p) < (1ull << 31), RSWA_ERR_UNSUPPORTED,
                  "attn_bwd: rows * heads_q too large for the statistics workspace");
   }

@@ -52,7 +52,8 @@ template <int D>
 struct DkvCfg {
   static constexpr int BM = 32;        // query rows per step
   static constexpr int KB = 2;         // 32-key blocks per wave
-  static constexpr int BN = 256;       // keys per block: 4 waves x KB x 32
+  static constexpr int BN = kDkvKeysPerBlock;  // keys per block: 4 waves x KB x 32
+  static_assert(BN == 256, "4 waves x KB x 32 keys");
   static constexpr int THREADS = 256;  // one wave per SIMD, up to 512 registers each
   static constexpr int KSTEPS = D / 16;
   static constexpr int DBLK = D / 32;
@@ -62,7 +63,7 @@ struct DkvCfg {
   static constexpr int V_TILE = BN * ROWB;
 };
 
-template <typename T, int D>
+template <typename T, int D, bool SPLIT>
 __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   using C = DkvCfg<D>;
   using M = Mma<T>;
@@ -75,6 +76,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   __shared__ __attribute__((aligned(1024))) char do_s1[C::Q_TILE];
   __shared__ __attribute__((aligned(1024))) float st_s0[2 * C::BM];  // -lse2[BM], -delta[BM]
   __shared__ __attribute__((aligned(1024))) float st_s1[2 * C::BM];
+  __shared__ int arrived_s;
 
   const int wid = logical_block_id(a.n_work);
   if (wid < 0) return;
@@ -86,9 +88,13 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   const int i16 = lane & 15;
   const int u = lane >> 4;
 
-  // ---- which (sequence, kv head, key tile) ---------------------------------
-  const int slot = a.rev_k ? a.n_tile - 1 - wid % a.n_tile : wid % a.n_tile;
-  int rest = wid / a.n_tile;
+  // ---- which (sequence, kv head, key tile) and which part of the GQA group -----------
+  // parts of a tile are neighbours in the launch order; tiles go heaviest first
+  const int part = wid % a.nsplit;
+  const int unit = wid / a.nsplit;
+  const int hpu = a.group / a.nsplit;  // q heads this block walks
+  const int slot = a.rev_k ? a.n_tile - 1 - unit % a.n_tile : unit % a.n_tile;
+  int rest = unit / a.n_tile;
   const int hk = rest % a.heads_kv;
   SeqInfo s;
   int kt;
@@ -120,7 +126,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
       (a.wl >= 0 && j0 >= a.n_sink) ? min(len_q - 1, j_last - shift + a.wl) : len_q - 1;
   const int qt_lo = i_min / C::BM;
   const int n_qt = (i_max >= i_min) ? i_max / C::BM - qt_lo + 1 : 0;
-  const int n_iter = n_qt * a.group;
+  const int n_iter = n_qt * hpu;
 
   const int jw0 = j0 + wave * (32 * KB);  // first key column of this wave
   const int jw1 = jw0 + 32 * KB - 1;
@@ -199,9 +205,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   nxt.qt = qt_start;
   nxt.i0 = i_first + qt_start * C::BM;
   int nxt_left = n_qt;  // tiles left in the walk of nxt's head, nxt included
-  nxt.q_head = q_base + (int64_t)hk * a.group * a.q_st[2];
-  nxt.do_head = do_base + (int64_t)hk * a.group * a.do_st[2];
-  nxt.stat_row = (int64_t)hk * a.group * a.rows_q + ws_row0;
+  const int h_first = hk * a.group + part * hpu;
+  nxt.q_head = q_base + (int64_t)h_first * a.q_st[2];
+  nxt.do_head = do_base + (int64_t)h_first * a.do_st[2];
+  nxt.stat_row = (int64_t)h_first * a.rows_q + ws_row0;
   // The next tile is fetched by NPART instructions per wave (statistics, Q, dO), issued
   // one at a time between the first MFMAs of a step; advance() then moves the cursor on.
   constexpr int NQD = TileDma<D, C::BM, C::THREADS>::N;
@@ -425,25 +432,84 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   int lane_e = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
   asm volatile("" : "+v"(lane_e));
   const int l32_e = lane_e & 31, g_e = lane_e >> 5;
-#pragma unroll
-  for (int kb = 0; kb < KB; kb++) {
+  // value group (mtx: 0 dK / 1 dV, key block, d block, four consecutive d) of this lane -> memory
+  auto emit = [&](int mtx, int kb, int d, int i4, f32x4 val) __attribute__((always_inline)) {
     const int jc = jw0 + kb * 32 + l32_e;
     if (jc < len_k) {
+      const float sc = mtx == 0 ? a.scale : 1.f;
+      T* dst = mtx == 0 ? dk_ptr + (int64_t)jc * a.dk_st[1] : dv_ptr + (int64_t)jc * a.dv_st[1];
+      *(typename M::V4*)(dst + d * 32 + 8 * i4 + 4 * g_e) =
+          M::pack4(val[0] * sc, val[1] * sc, val[2] * sc, val[3] * sc);
+    }
+  };
+  // Without a split (SPLIT = false, nsplit = 1) the lane's sums go straight out.  Otherwise the
+  // group's q heads were dealt to nsplit blocks: every block stores its fp32 partial sums (16
+  // bytes per lane and value group, lanes contiguous), then counts itself in; the block that
+  // arrives last adds the parts in part order -- the same order whichever block that is, so
+  // the result does not depend on timing -- and writes dK, dV.  Nobody waits for anybody.
+  constexpr int GROUPS = 2 * KB * DB * 4;  // value groups per lane
+  f32x4* part_base = (f32x4*)a.dkv_part + (int64_t)unit * a.nsplit * (GROUPS * C::THREADS);
+  {
+    // one running pointer (opaque to the optimiser, or it would keep 64 addresses in registers)
+    f32x4* mine = part_base + (int64_t)part * (GROUPS * C::THREADS) + (wave * 64 + lane_e);
 #pragma unroll
-      for (int mtx = 0; mtx < 2; mtx++) {  // 0: dK, 1: dV
-        const float sc = mtx == 0 ? a.scale : 1.f;
-        T* dst = mtx == 0 ? dk_ptr + (int64_t)jc * a.dk_st[1] : dv_ptr + (int64_t)jc * a.dv_st[1];
+    for (int mtx = 0; mtx < 2; mtx++)
+#pragma unroll
+      for (int kb = 0; kb < KB; kb++)
 #pragma unroll
         for (int d = 0; d < DB; d++)
 #pragma unroll
           for (int i4 = 0; i4 < 4; i4++) {
             const f32x16& acc = mtx == 0 ? dk_acc[kb][d] : dv_acc[kb][d];
-            const auto h4 = M::pack4(acc[4 * i4] * sc, acc[4 * i4 + 1] * sc, acc[4 * i4 + 2] * sc,
-                                     acc[4 * i4 + 3] * sc);
-            *(typename M::V4*)(dst + d * 32 + 8 * i4 + 4 * g_e) = h4;
+            const f32x4 val = {acc[4 * i4], acc[4 * i4 + 1], acc[4 * i4 + 2], acc[4 * i4 + 3]};
+            if constexpr (!SPLIT) {
+              emit(mtx, kb, d, i4, val);
+            } else {
+              *mine = val;
+              mine += C::THREADS;
+              asm volatile("" : "+v"(mine));
+            }
           }
+  }
+  if constexpr (!SPLIT) return;
+  // Release: every wave waits for its own stores, then one thread makes the block's partial
+  // sums visible device-wide and counts the block in.  Acquire on the other side: the block
+  // that finds itself last drops what its compute unit and L2 may hold of those lines.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  if (tid == 0) {
+    __threadfence();
+    arrived_s = atomicAdd(a.dkv_count + unit, 1);
+  }
+  __syncthreads();
+  if (arrived_s != a.nsplit - 1) return;
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+  if (tid == 0) a.dkv_count[unit] = 0;  // the next launch on this workspace starts from zero
+  // eight value groups at a time, all their loads in flight before the first sum
+  const f32x4* parts = part_base + (wave * 64 + lane_e);
+  constexpr int GB = 8;
+  static_assert(GROUPS % GB == 0, "batches of value groups");
+  for (int g0 = 0; g0 < GROUPS; g0 += GB) {  // group = ((mtx KB + kb) DB + d) 4 + i4
+    // four loads per group whatever nsplit is (a part past the last reads the last one again
+    // and is left out of the sum): no branch, so nothing waits between the loads
+    f32x4 v[GB][4];
+#pragma unroll
+    for (int j = 0; j < GB; j++)
+#pragma unroll
+      for (int pp = 0; pp < 4; pp++)
+        v[j][pp] = parts[(int64_t)min(pp, a.nsplit - 1) * (GROUPS * C::THREADS) + j * C::THREADS];
+#pragma unroll
+    for (int j = 0; j < GB; j++) {
+      f32x4 sum = v[j][0];
+#pragma unroll
+      for (int pp = 1; pp < 4; pp++) {
+        const float use = pp < a.nsplit ? 1.f : 0.f;
+        sum += v[j][pp] * use;
       }
+      const int grp = g0 + j;
+      emit(grp / (KB * DB * 4), grp / (DB * 4) % KB, grp / 4 % DB, grp % 4, sum);
     }
+    parts += GB * C::THREADS;
   }
 }
 
@@ -727,6 +793,9 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(const AttnArgs a) {
 template <typename T, int D>
 __global__ __launch_bounds__(256) void attn_bwd_prep_kernel(const AttnArgs a) {
   constexpr int LPR = D / 8;
+  // arrival counters of the dK/dV kernel's split blocks start from zero
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < a.n_count; i += (int64_t)gridDim.x * 256)
+    a.dkv_count[i] = 0;
   const int64_t unit = ((int64_t)blockIdx.x * 256 + threadIdx.x) / LPR;  // (row, head)
   const int c = (threadIdx.x % LPR) * 8;
   if (unit >= a.rows_q * a.heads_q) return;
@@ -771,7 +840,8 @@ __global__ __launch_bounds__(256) void attn_bwd_prep_kernel(const AttnArgs a) {
 // Explicit instantiations: with implicit instantiation alone this hipcc emits the host
 // launch stubs of only some of the variants.
 #define RSWA_INSTANTIATE(T, D)                                              \
-  template __global__ void attn_bwd_dkdv_kernel<T, D>(const AttnArgs);      \
+  template __global__ void attn_bwd_dkdv_kernel<T, D, false>(const AttnArgs); \
+  template __global__ void attn_bwd_dkdv_kernel<T, D, true>(const AttnArgs);  \
   template __global__ void attn_bwd_dq_kernel<T, D>(const AttnArgs);        \
   template __global__ void attn_bwd_prep_kernel<T, D>(const AttnArgs);
 RSWA_INSTANTIATE(__bf16, 128)
@@ -792,17 +862,23 @@ int launch_bwd(AttnArgs& a, hipStream_t stream, int phases) {
   }
   if (phases & RSWA_BWD_DKDV) {
     using C = DkvCfg<D>;
+    if (a.rows_q == 0) a.nsplit = 1;  // nothing to walk (and no statistics launch ran)
     if (a.cu_q) {
       a.n_tile = (int)(ceil_div(a.rows_k, C::BN) + a.batch);
-      a.n_work = a.n_tile * a.heads_kv;
+      a.n_work = a.n_tile * a.heads_kv * a.nsplit;
     } else {
       a.n_tile = (int)ceil_div(a.seqlen_k, C::BN);
-      a.n_work = a.n_tile * a.heads_kv * a.batch;
+      a.n_work = a.n_tile * a.heads_kv * a.batch * a.nsplit;
     }
     if (a.n_work > 0) {
       clear_launch_error();
-      hipLaunchKernelGGL((attn_bwd_dkdv_kernel<T, D>), dim3(padded_grid(a.n_work)),
-                         dim3(C::THREADS), 0, stream, a);
+      if (a.nsplit > 1) {
+        hipLaunchKernelGGL((attn_bwd_dkdv_kernel<T, D, true>), dim3(padded_grid(a.n_work)),
+                           dim3(C::THREADS), 0, stream, a);
+      } else {
+        hipLaunchKernelGGL((attn_bwd_dkdv_kernel<T, D, false>), dim3(padded_grid(a.n_work)),
+                           dim3(C::THREADS), 0, stream, a);
+      }
       int rc = check_launch("attn_bwd dkdv");
       if (rc != RSWA_OK) return rc;
     }
@@ -833,10 +909,11 @@ int launch_bwd(AttnArgs& a, hipStream_t stream, int phases) {
 }  // namespace
 }  // namespace rswa
 
-extern "C" int rswa_attn_bwd_phases(const rswa_attn_params* p, void* stream, int phases) {
-  using namespace rswa;
+namespace rswa {
+namespace {
+int bwd_entry(const rswa_attn_params* p, void* stream, int phases, bool allow_split) {
   AttnArgs a;
-  int rc = fill_args(p, true, a);
+  int rc = fill_args(p, true, a, allow_split);
   if (rc != RSWA_OK) return rc;
   hipStream_t st = (hipStream_t)stream;
   if (p->dtype == RSWA_BF16) {
@@ -845,6 +922,12 @@ extern "C" int rswa_attn_bwd_phases(const rswa_attn_params* p, void* stream, int
   }
   return p->head_dim == 128 ? launch_bwd<_Float16, 128>(a, st, phases)
                             : launch_bwd<_Float16, 64>(a, st, phases);
+}
+}  // namespace
+}  // namespace rswa
+
+extern "C" int rswa_attn_bwd_phases(const rswa_attn_params* p, void* stream, int phases) {
+  return rswa::bwd_entry(p, stream, phases, true);
 }
 
 extern "C" int rswa_attn_bwd(const rswa_attn_params* p, void* stream) {
@@ -889,7 +972,8 @@ void* scratch_on_current_device() {
 extern "C" int rswa_attn_bwd_static(const rswa_attn_params* p, void* stream) {
   using namespace rswa;
   RSWA_REQUIRE(p != nullptr, RSWA_ERR_INVALID, "attn_bwd_static: null params");
-  const uint64_t need = rswa_attn_bwd_workspace_bytes(p);
+  // statistics only: on the built-in buffer the dK/dV kernel never splits its key tiles
+  const uint64_t need = bwd_layout(p, false).total_bytes;
   RSWA_REQUIRE(need <= RSWA_BWD_STATIC_MAX_BYTES, RSWA_ERR_UNSUPPORTED,
                "attn_bwd_static: rows * heads_q needs %llu bytes of statistics, the built-in "
                "buffer holds %llu (use rswa_attn_bwd with a caller workspace)",
@@ -901,11 +985,11 @@ extern "C" int rswa_attn_bwd_static(const rswa_attn_params* p, void* stream) {
   q.workspace_bytes = RSWA_BWD_STATIC_MAX_BYTES;
   {
     AttnArgs probe;
-    int rc = fill_args(&q, true, probe);
+    int rc = fill_args(&q, true, probe, false);
     if (rc != RSWA_OK) return rc;
   }
   void* ptr = scratch_on_current_device();
   if (!ptr) return RSWA_ERR_LAUNCH;
   q.workspace = ptr;
-  return rswa_attn_bwd(&q, stream);
+  return bwd_entry(&q, stream, RSWA_BWD_PREP | RSWA_BWD_DKDV | RSWA_BWD_DQ, false);
 }

@@ -34,6 +34,12 @@ struct AttnArgs {
   void* dv;
   float* delta;   // fp32 [heads_q, rows_q] packed: -sum_d dO * O         (workspace)
   float* lse2;    // fp32 [heads_q, rows_q] packed: -lse * log2(e); empty rows -inf (workspace)
+  // dK/dV kernel with the q heads of a GQA group split over `nsplit` blocks per key tile:
+  // fp32 partial sums [tile unit][part] and one arrival counter per tile unit (workspace)
+  float* dkv_part;
+  int32_t* dkv_count;
+  int32_t nsplit;     // 1: one block per (key tile, kv head) walks the whole group
+  int32_t n_count;    // arrival counters in the workspace
   const int32_t* cu_q;
   const int32_t* cu_k;
   int64_t q_st[3], k_st[3], v_st[3], o_st[3], do_st[3], dq_st[3], dk_st[3], dv_st[3], lse_st[3];
@@ -294,7 +300,33 @@ __device__ __forceinline__ float halfwave_sum(float x) {
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
+// Keys per block of the dK/dV kernel, and how a launch of it is laid out: with so few key
+// tiles that one block per (tile, kv head) would leave half of the 256 compute units without
+// work, the q heads of each GQA group are dealt to `nsplit` blocks, whose fp32 partial sums
+// meet in the workspace.  Measured on the rank share (8192-token chunk, window 4096, 32 / 8
+// heads): the previous-chunk corner (128 blocks) 0.75 -> 0.30 ms; the own-chunk block (256
+// blocks of 32..544 steps) gains 4 % alone and loses 8 % beside the corner launch -- more
+// compute units busy lowers the shader clock (1.92 -> 1.77 GHz), and every part pays its own
+// prologue, partial store and share of the final sum -- so launches that already give every
+// compute unit a block are left alone.
+constexpr int kDkvKeysPerBlock = 256;
+constexpr int kComputeUnits = 256;  // MI355X
+#ifndef RSWA_DKDV_SPLIT_BELOW
+#define RSWA_DKDV_SPLIT_BELOW (kComputeUnits / 2 + 1)
+#endif
+constexpr int kDkvSplitBelow = RSWA_DKDV_SPLIT_BELOW;  // split launches of fewer blocks
+struct BwdLayout {
+  uint64_t stats_bytes;    // each of the two statistics arrays
+  int nsplit;
+  int n_tile_k;            // key tile slots per kv head (dense: per batch entry)
+  int n_count;             // arrival counters (one per key tile unit)
+  uint64_t count_off, part_off, total_bytes;
+};
+BwdLayout bwd_layout(const rswa_attn_params* p, bool allow_split);
+
 // Fill an AttnArgs from the public struct; validates what both directions share.
-int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a);
+// `allow_split` = false keeps the dK/dV kernel at one block per key tile, whatever the shape
+// (workspace holds the statistics only).
+int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a, bool allow_split = true);
 
 }  // namespace rswa

@@ -153,7 +153,7 @@ def attn_bwd(
 ) -> None:
     """Masked attention backward; overwrites ``dq, dk, dv`` (views are fine).
 
-    ``workspace`` (uint8, at least ``bwd_workspace_bytes(q)``) may be supplied to avoid the
+    ``workspace`` (uint8, at least ``bwd_workspace_bytes(q, k, ...)``) may be supplied to avoid the
     per-call scratch allocation, and must be when the phases of one backward are spread
     over several calls; ``phases`` is the bit mask of ``rswa_attn_bwd_phases`` (1 prep,
     2 dk/dv kernel, 4 dq kernel).  ``dq_accumulate`` adds this call's dQ to the values
@@ -216,11 +216,15 @@ def attn_bwd(
         _lib.check(L.rswa_attn_bwd_phases(p, _lib.stream_ptr(dev), int(phases)))
 
 
-def bwd_workspace_bytes(q: torch.Tensor) -> int:
-    """Scratch size of one backward over the rows of ``q`` (dense ``[B,S,H,D]`` or packed
-    ``[T,H,D]``): two fp32 values per (row, head), as ``rswa_attn_bwd_workspace_bytes``
-    computes it, plus alignment slack."""
-    return (q.numel() // q.shape[-1]) * 8 + 1024
+def bwd_workspace_bytes(q: torch.Tensor, k: torch.Tensor,
+                        cu_seqlens_q: Optional[torch.Tensor] = None,
+                        cu_seqlens_k: Optional[torch.Tensor] = None) -> int:
+    """Scratch size of one backward over ``q`` against ``k`` (dense ``[B,S,H,D]`` or packed
+    ``[T,H,D]``), as ``rswa_attn_bwd_workspace_bytes`` computes it: two fp32 values per
+    (row, q head), plus the partial sums of the dK/dV kernel when the shape makes it deal the
+    q heads of a GQA group to several blocks."""
+    p = _params(q, k, k, 1.0, (-1, -1), False, cu_seqlens_q, cu_seqlens_k, 0)
+    return int(_lib.lib().rswa_attn_bwd_workspace_bytes(p))
 
 
 # ---- names of the upstream wrappers -----------------------------------------

@@ -278,9 +278,14 @@ def _backward_two_blocks(q, k, v, prev_kv, out, lse, do, plan, scale, local_cu):
     (_, _, _, window0, causal0), (i1, qs, ks, window1, causal1) = plan
     dq, dk, dv = torch.zeros_like(q), torch.empty_like(k), torch.empty_like(v)
     dprev = [torch.zeros_like(kv) for kv in prev_kv]
-    ws = torch.empty(bwd_workspace_bytes(q), dtype=torch.uint8, device=q.device)
-    ws_prev = torch.empty(bwd_workspace_bytes(q[:, qs]), dtype=torch.uint8, device=q.device)
     kk, vv, dkv = prev_kv[i1 - 1][0], prev_kv[i1 - 1][1], dprev[i1 - 1]
+    if local_cu is not None:
+        need = bwd_workspace_bytes(q[0], k[0], local_cu, local_cu)
+    else:
+        need = bwd_workspace_bytes(q, k)
+    ws = torch.empty(need, dtype=torch.uint8, device=q.device)
+    ws_prev = torch.empty(bwd_workspace_bytes(q[:, qs], kk[:, ks]), dtype=torch.uint8,
+                          device=q.device)
 
     def own(phases, accumulate):
         if local_cu is not None:

@@ -238,7 +238,7 @@ def test_bwd_dq_accumulate_is_one_fp32_add_of_the_two_16bit_values(hq, hk, s):
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     attn_bwd(q, k, v, out, lse, do, dq, dk, dv, None, (100, 0), True)
     acc, dk2, dv2 = base.clone(), torch.empty_like(k), torch.empty_like(v)
-    ws = torch.empty(bwd_workspace_bytes(q), dtype=torch.uint8, device="cuda")
+    ws = torch.empty(bwd_workspace_bytes(q, k), dtype=torch.uint8, device="cuda")
     attn_bwd(q, k, v, out, lse, do, acc, dk2, dv2, None, (100, 0), True, workspace=ws, phases=3)
     assert torch.equal(acc, base)  # the dQ kernel has not run yet
     attn_bwd(q, k, v, out, lse, do, acc, dk2, dv2, None, (100, 0), True, workspace=ws, phases=4,

@@ -1,6 +1,6 @@
 """The allocation-free backward entry point (``rswa_attn_bwd_static``, statistics in the
-library's own device buffer) gives bit for bit what ``rswa_attn_bwd`` gives with a caller
-workspace: same kernels, same order.  Two calls in a row, the second on a smaller input, so
+library's own device buffer) gives what ``rswa_attn_bwd`` gives with a caller workspace: dQ
+bit for bit, dK / dV to the last place (see ``_same``).  Two calls in a row, the second on a smaller input, so
 that stale statistics of the first call would show; then a size beyond the buffer is refused.
 Collected last on purpose (file name): a failure here must not hide the other tests."""
 import pytest
@@ -37,19 +37,32 @@ def _both(q, k, v, do, window, cu=None):
     return grads
 
 
+def _same(with_workspace, static):
+    """dQ bit for bit.  dK / dV: with a caller workspace the dK/dV kernel may deal the q heads of
+    a GQA group to several blocks and add their fp32 partial sums at the end; on the built-in
+    buffer it never does, so the fp32 sums are associated differently and the 16-bit results
+    may differ in the last place of single entries (floating point: the path's tolerance is a
+    relative norm of 5e-2; asserted here: one 16-bit unit in the last place)."""
+    assert torch.equal(with_workspace[0], static[0])
+    for x, y in zip(with_workspace[1:], static[1:]):
+        assert not torch.isnan(y.float()).any()
+        x, y = x.float(), y.float()
+        # one unit in the last place of the entry, plus the fp32 reassociation error of sums
+        # whose terms are as large as the tensor's largest entry (entries that nearly cancel)
+        ulp = torch.maximum(x.abs(), y.abs()) * 2.0 ** -7 + 4e-6 * x.abs().max()
+        assert ((x - y).abs() <= ulp).all()
+        assert (x != y).float().mean().item() < 0.05
+
+
 def test_static_backward_equals_workspace_backward_twice_in_a_row():
     # first call: 2 x 1536 rows x 8 heads; second, smaller: packed 700 rows x 4 heads
     q, k, v, do = _case(0, 2, 1536, 8, 2, 128, (200, 0))
     (a, b) = _both(q, k, v, do, (200, 0))
-    for x, y in zip(a, b):
-        assert not torch.isnan(y.float()).any()
-        assert torch.equal(x, y)
+    _same(a, b)
     cu = torch.tensor([0, 130, 131, 500, 700], dtype=torch.int32, device="cuda")
     q, k, v, do = _case(1, 1, 700, 4, 4, 64, (64, 0), packed_cu=cu)
     (a, b) = _both(q, k, v, do, (64, 0), cu)
-    for x, y in zip(a, b):
-        assert not torch.isnan(y.float()).any()
-        assert torch.equal(x, y)
+    _same(a, b)
 
 
 def test_static_backward_refuses_sizes_beyond_its_buffer():
