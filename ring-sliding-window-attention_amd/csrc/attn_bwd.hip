@@ -14,9 +14,10 @@
 //          256 rows of one head) walks the key tiles (64 keys) it can see, like the forward
 //          kernel; dQ^T stays in registers
 // S and dP are computed in both main kernels (7 GEMM units instead of 5).  That costs
-// less here than fp32 atomics on dQ: the L2 retires about one fp32 atomic per clock per
-// channel, which caps an atomic dQ far below the MFMA rate.  It also makes the result
-// run-to-run deterministic.
+// less here than fp32 atomics on dQ: hardware fp32 atomic adds retire at 340 G elements/s on
+// the whole device (measured with 64 consecutive floats per wave instruction, the pattern a
+// fused kernel would use), a dQ tile of 32 x 128 per 256-key block and step needs 700 G/s at
+// the rate the dK/dV kernel walks.  It also makes the result run-to-run deterministic.
 //
 // DKDV per (query tile, wave) (C layout: lane = key; two 32-key blocks per wave, so every
 // fragment read from LDS feeds two MFMAs):
@@ -30,9 +31,11 @@
 // the code keeps at least two later MFMAs between the last one that writes S or dP and
 // the first read of the result.  The dK^T / dV^T MFMAs are compiler builtins (accumulation
 // registers), so every copy or read the compiler adds around them is padded as required.
-// DQ per (key tile, wave); wave owns 32 query columns (C layout: lane = query):
-//   S^T = K Q^T, dP^T = V dO^T  A = K / V row fragments from LDS, B = Q / dO fragments (regs)
-//   dS^T as above with per-lane lse2 / delta
+// DQ per (key tile, wave), on 16x16x32 MFMAs; wave owns 32 query columns (lane = query l % 16
+// of two 16-query blocks):
+//   S^T = K Q^T, dP^T = V dO^T  A = K / V row fragments from LDS, B = Q c / dO fragments (regs);
+//                               the chains start from -lse2 / -delta of the lane's queries
+//   dS^T = exp2(S^T) dP^T       (one exponential, one product, the 16-bit conversion per score)
 //   dQ^T += K^T dS^T            A = transposing LDS reads of K, B = dS^T (regs)
 //
 // Streamed tiles are double-buffered in SEPARATE static __shared__ arrays, filled by buffer
@@ -516,12 +519,22 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
 // ============================================================================
 // dQ
 // ============================================================================
+// LDS read-ahead of the dQ kernel's two matrix sections, in fragments (measured: 8 / 4 is
+// 2-3 % faster than 6 / 4 and than 12 / 6; the register file, all 256 registers of a lane
+// at head_dim 128, allows no more in the first section once S^T and dP^T are both live)
+#ifndef RSWA_DQ_AH1
+#define RSWA_DQ_AH1 8
+#endif
+#ifndef RSWA_DQ_AH2
+#define RSWA_DQ_AH2 4
+#endif
 template <int D>
 struct DqCfg {
   static constexpr int BN = 64;  // keys per step
   static constexpr int THREADS = 512;
-  static constexpr int KSTEPS = D / 16;
-  static constexpr int DBLK = D / 32;
+  static constexpr int KS = D / 32;   // k-steps of the 16x16x32 MFMAs over the head dim
+  static constexpr int DB = D / 16;   // 16-row blocks of dQ^T
+  static constexpr int KBLK = BN / 16;  // 16-key blocks per tile
   static constexpr int CPR = D / 8;
   static constexpr int ROWB = D * 2;
   static constexpr int TILE = BN * ROWB;
@@ -529,11 +542,20 @@ struct DqCfg {
   static_assert(TILE >= 32 * O_STRIDE, "one wave's epilogue staging fits one tile buffer");
 };
 
+// Built on v_mfma_f32_16x16x32 (with random operands the matrix pipes sustain about 14 % more
+// of these than of the 32x32x16 form before the power limit pulls the clock down).  A wave
+// owns 32 query rows as two 16-column blocks: lane l holds query column l % 16 of each block;
+// its 8-element fragments cover d = 32 ks + 8 (l / 16) ...; a 64-key tile is four 16-key
+// blocks, and S^T / dP^T tiles hold keys 16 kb + 4 (l / 16) + i in element i.  Two such tiles
+// of neighbouring key blocks, packed, are the B operand of dQ^T += K^T dS^T over a 32-key slab
+// (k order: four keys of the first block, then four of the second); the A operand follows the
+// same order: two transposing reads, one per key block.
 template <typename T, int D>
 __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(const AttnArgs a) {
   using C = DqCfg<D>;
   using M = Mma<T>;
   using V8 = typename M::V8;
+  constexpr int KS = C::KS, DB = C::DB, KBLK = C::KBLK;
   __shared__ __attribute__((aligned(1024))) char k_s0[C::TILE];
   __shared__ __attribute__((aligned(1024))) char k_s1[C::TILE];
   __shared__ __attribute__((aligned(1024))) char v_s0[C::TILE];
@@ -544,10 +566,8 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(const AttnArgs a) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int l32 = lane & 31;
-  const int g = lane >> 5;
-  const int i16 = lane & 15;
-  const int u = lane >> 4;
+  const int r = lane & 15;   // column (query) / row (key, d) inside a 16 block
+  const int u = lane >> 4;   // k group
 
   // pair mode: waves 0-3 and 4-7 take the same 128 rows of two neighbouring q heads;
   // row mode: the 8 waves take 256 consecutive rows of one q head
@@ -596,47 +616,65 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(const AttnArgs a) {
   auto tile_of = [&](int it) { return it < n_sink_t ? it : t_lo + (it - n_sink_t); };
 
   const int r0 = i0 + (pair ? wave & 3 : wave) * 32;
-  const int iq = r0 + l32;
   const bool wave_valid = r0 < len_q;
   const bool wave_rows_full = r0 + 31 < len_q;
   const RowBounds wb_first = row_bounds(a, r0, len_q, len_k);
   const RowBounds wb_last = row_bounds(a, min(r0 + 31, len_q - 1), len_q, len_k);
 
-  // Q / dO fragments (B operands): lane = query column, 8 consecutive d per k-step
-  V8 qf[C::KSTEPS], dof[C::KSTEPS];
-  float lse2 = -__builtin_inff(), delta = 0.f;  // negated, as the workspace holds them
-  if (iq < len_q) {
+  // Q / dO fragments (B operands) and the statistics of the lane's two query rows.  Q is
+  // multiplied by scale * log2(e) here, once, and the (negated) statistics are the values the
+  // S^T and dP^T accumulator chains start from: the MFMAs then deliver S c - lse2 and
+  // dP - delta, and the vector ALU is left with one exponential, one product and the 16-bit
+  // conversion per score.  Rounding the scaled Q to 16 bits moves a score by about 2^-9 of its
+  // typical magnitude (P by about 0.1 %), a quarter of what rounding P itself to 16 bits does.
+  V8 qf[2][KS], dof[2][KS];
+  f32x4 lse2[2], delta[2];  // the row's value in all four elements
 #pragma unroll
-    for (int ks = 0; ks < C::KSTEPS; ks++) {
-      qf[ks] = *(const V8*)(q_ptr + (int64_t)iq * a.q_st[1] + ks * 16 + g * 8);
-      dof[ks] = *(const V8*)(do_ptr + (int64_t)iq * a.do_st[1] + ks * 16 + g * 8);
-    }
-    lse2 = a.lse2[(int64_t)hq * a.rows_q + ws_row0 + iq];
-    delta = a.delta[(int64_t)hq * a.rows_q + ws_row0 + iq];
-  } else {
+  for (int qb = 0; qb < 2; qb++) {
+    const int iq = r0 + 16 * qb + r;
+    float l2 = -__builtin_inff(), dl = 0.f;
+    if (iq < len_q) {
 #pragma unroll
-    for (int ks = 0; ks < C::KSTEPS; ks++) {
-      qf[ks] = V8{0, 0, 0, 0, 0, 0, 0, 0};
-      dof[ks] = V8{0, 0, 0, 0, 0, 0, 0, 0};
+      for (int ks = 0; ks < KS; ks++) {
+        const V8 qraw = *(const V8*)(q_ptr + (int64_t)iq * a.q_st[1] + ks * 32 + u * 8);
+        float qs[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) qs[j] = (float)qraw[j] * a.scale_log2;
+        qf[qb][ks] = M::pack(qs);
+        dof[qb][ks] = *(const V8*)(do_ptr + (int64_t)iq * a.do_st[1] + ks * 32 + u * 8);
+      }
+      l2 = a.lse2[(int64_t)hq * a.rows_q + ws_row0 + iq];
+      dl = a.delta[(int64_t)hq * a.rows_q + ws_row0 + iq];
+    } else {
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++) {
+        qf[qb][ks] = V8{0, 0, 0, 0, 0, 0, 0, 0};
+        dof[qb][ks] = V8{0, 0, 0, 0, 0, 0, 0, 0};
+      }
     }
+    lse2[qb] = f32x4{l2, l2, l2, l2};
+    delta[qb] = f32x4{dl, dl, dl, dl};
   }
 
-  f32x16 dq_acc[C::DBLK];
+  f32x4 dq_acc[DB][2];
 #pragma unroll
-  for (int d = 0; d < C::DBLK; d++)
+  for (int d = 0; d < DB; d++)
 #pragma unroll
-    for (int i = 0; i < 16; i++) dq_acc[d][i] = 0.f;
+    for (int qb = 0; qb < 2; qb++) dq_acc[d][qb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  // lane-constant LDS offsets (see the forward kernel)
-  const int a_row = l32 * C::ROWB + ((g ^ swz_f<C::CPR>(l32)) << 4);
-  const int rl = 4 * g + (i16 >> 2);
-  const int lp = 2 * (u & 1) + ((i16 & 3) >> 1);
-  const int t_row0 = rl * C::ROWB + ((lp ^ swz_f<C::CPR>(rl)) << 4) + (i16 & 1) * 8;
-  const int t_row1 = (rl + 8) * C::ROWB + ((lp ^ swz_f<C::CPR>(rl + 8)) << 4) + (i16 & 1) * 8;
+  // ---- lane-constant LDS offsets (swizzle folded: the varying parts are XOR / immediates) ----
+  // row fragments of K / V (16-byte reads): row 16 kb + r, chunk 4 ks + u
+  //   offset = (a_row ^ (ks << 6)) + kb * 16 * ROWB
+  const int a_row = r * C::ROWB + ((u ^ swz16_f<C::CPR>(r)) << 4);
+  // transposing reads of K: row 32 ks2 + 16 blk + 4 u + (r >> 2), chunk 2 db + ((r & 3) >> 1),
+  // second half of the chunk for odd r
+  //   offset = (t_row ^ (db << 5)) + (32 ks2 + 16 blk) * ROWB
+  const int rl = 4 * u + (r >> 2);
+  const int t_row = rl * C::ROWB + ((((r & 3) >> 1) ^ swz16_f<C::CPR>(rl)) << 4) + (r & 1) * 8;
 
   const __amdgpu_buffer_rsrc_t k_rsrc = make_rows_rsrc(k_ptr, len_k, a.k_st[1] * 2, C::ROWB);
   const __amdgpu_buffer_rsrc_t v_rsrc = make_rows_rsrc(v_ptr, len_k, a.v_st[1] * 2, C::ROWB);
-  TileDma<D, C::BN, C::THREADS> k_dma, v_dma;
+  TileDma<D, C::BN, C::THREADS, true> k_dma, v_dma;
   k_dma.init(a.k_st[1], tid);
   v_dma.init(a.v_st[1], tid);
   const int k_tile_bytes = (int)(C::BN * a.k_st[1] * 2), v_tile_bytes = (int)(C::BN * a.v_st[1] * 2);
@@ -653,89 +691,107 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(const AttnArgs a) {
     const bool needed =
         wave_valid && j0 <= wb_last.hi && (j1 >= wb_first.lo || j0 < a.n_sink);
     if (needed) {
-      // S^T = K Q^T and dP^T = V dO^T (rows = keys, lane = query column)
-      f32x16 sacc[2], pacc[2];
-#pragma unroll
-      for (int t = 0; t < 2; t++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-          sacc[t][i] = 0.f;
-          pacc[t][i] = 0.f;
-        }
-#pragma unroll
-      for (int ks = 0; ks < C::KSTEPS; ks++) {
-        const int off = a_row ^ (ks << 5);
-#pragma unroll
-        for (int t = 0; t < 2; t++) {
-          sacc[t] = M::mfma32(*(const V8*)(kc + off + t * 32 * C::ROWB), qf[ks], sacc[t]);
-          pacc[t] = M::mfma32(*(const V8*)(vc + off + t * 32 * C::ROWB), dof[ks], pacc[t]);
-        }
-      }
-      // LDS reads eight fragments ahead of the MFMAs that use them
-      __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
-#pragma unroll
-      for (int i = 0; i < 4 * C::KSTEPS - 8; i++) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      }
-      __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
       const bool full = wave_rows_full && j1 <= wb_first.hi &&
                         (j0 >= wb_last.lo || j1 < a.n_sink);
-      if (full) {
+      // S^T and dP^T (element i of tile [kb][qb]: key 16 kb + 4 u + i, query 16 qb + r); every
+      // K / V fragment read feeds the MFMAs of both query blocks; the chains start from the
+      // row statistics.  The two waves of a SIMD overlap best when each keeps its matrix and
+      // its vector work apart: vector instructions placed between a wave's own MFMAs hold its
+      // MFMAs back, the other wave's do not.
+      f32x4 sacc[KBLK][2], pacc[KBLK][2];
+      // (the lane offset is made opaque here: its XOR variants, times the buffers, would
+      // otherwise be kept in registers across the whole loop)
+      int a_off = a_row;
+      asm volatile("" : "+v"(a_off));
 #pragma unroll
-        for (int t = 0; t < 2; t++)
+      for (int ks = 0; ks < KS; ks++)
 #pragma unroll
-          for (int i = 0; i < 16; i++) {
-            const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[t][i], a.scale_log2, lse2));
-            pacc[t][i] = p * (pacc[t][i] + delta);
+        for (int kb = 0; kb < KBLK; kb++) {
+          const int off = (a_off ^ (ks << 6)) + kb * 16 * C::ROWB;
+          const V8 kfrag = *(const V8*)(kc + off);
+          const V8 vfrag = *(const V8*)(vc + off);
+#pragma unroll
+          for (int qb = 0; qb < 2; qb++) {
+            sacc[kb][qb] = M::mfma16(kfrag, qf[qb][ks], ks == 0 ? lse2[qb] : sacc[kb][qb]);
+            pacc[kb][qb] = M::mfma16(vfrag, dof[qb][ks], ks == 0 ? delta[qb] : pacc[kb][qb]);
           }
-      } else {
-        // edge tile: the lane's own mask bounds are recomputed here (only a few tiles per
-        // block take this path; kept across the loop they cost two registers, i.e. spills)
-        int lane_m = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
-        asm volatile("" : "+v"(lane_m));
-        const RowBounds rb = row_bounds(a, r0 + (lane_m & 31), len_q, len_k);
-        const int g_m = lane_m >> 5;
-        const int hi_rel = rb.hi - j0;
-        const int lo_rel = rb.lo - j0;
-        const int sink_rel = a.n_sink - j0;
-#pragma unroll
-        for (int t = 0; t < 2; t++)
-#pragma unroll
-          for (int i = 0; i < 16; i++) {
-            const int j = t * 32 + 8 * (i >> 2) + 4 * g_m + (i & 3);
-            const bool ok = (j <= hi_rel) & ((j >= lo_rel) | (j < sink_rel));
-            const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[t][i], a.scale_log2, lse2));
-            pacc[t][i] = ok ? p * (pacc[t][i] + delta) : 0.f;
-          }
-      }
-      // dQ^T[d, query] += K^T dS^T; dS^T is packed before the matrix section starts and the
-      // transposing reads run four fragments ahead of their MFMA
-      V8 dsb[4];
-#pragma unroll
-      for (int s4 = 0; s4 < 4; s4++) {
-        float dsv[8];
-#pragma unroll
-        for (int j = 0; j < 8; j++) dsv[j] = pacc[s4 >> 1][8 * (s4 & 1) + j];
-        dsb[s4] = M::pack(dsv);
-        asm volatile("" : "+v"(dsb[s4]));
-      }
-#pragma unroll
-      for (int s4 = 0; s4 < 4; s4++) {
-#pragma unroll
-        for (int d = 0; d < C::DBLK; d++) {
-          const int off0 = (t_row0 ^ (d << 6)) + s4 * 16 * C::ROWB;
-          const int off1 = (t_row1 ^ (d << 6)) + s4 * 16 * C::ROWB;
-          dq_acc[d] = M::mfma32(tr_pair<V8>(kc + off0, kc + off1), dsb[s4], dq_acc[d]);
         }
-      }
-      __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+      {
+        constexpr int NRD = 2 * KBLK * KS, AH = RSWA_DQ_AH1;  // LDS reads AH ahead, 2 MFMAs each
+        __builtin_amdgcn_sched_group_barrier(0x100, AH, 0);
 #pragma unroll
-      for (int i = 0; i < 4 * C::DBLK - 4; i++) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        for (int i = 0; i < NRD - AH; i++) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 2 * AH, 0);
       }
-      __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+      // P = exp2(S c - lse2), dS^T = P (dP^T - delta), packed slab by slab (32 keys) as the B
+      // operands of dQ^T += K^T dS^T
+      V8 dsb[2][2];
+      auto body = [&](auto full_c) __attribute__((always_inline)) {
+        constexpr bool FULL = decltype(full_c)::value;
+        int hi_rel[2], lo_rel[2], sink_rel = 0, u_m = 0;
+        if constexpr (!FULL) {
+          // edge tile: the lane's own mask bounds are recomputed here (only a few tiles per
+          // block take this path; kept across the loop they would cost registers)
+          int lane_m = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+          asm volatile("" : "+v"(lane_m));
+          u_m = lane_m >> 4;
+          sink_rel = a.n_sink - j0;
+#pragma unroll
+          for (int qb = 0; qb < 2; qb++) {
+            const RowBounds rb = row_bounds(a, r0 + 16 * qb + (lane_m & 15), len_q, len_k);
+            hi_rel[qb] = rb.hi - j0;
+            lo_rel[qb] = rb.lo - j0;
+          }
+        }
+#pragma unroll
+        for (int ks2 = 0; ks2 < 2; ks2++)
+#pragma unroll
+          for (int qb = 0; qb < 2; qb++) {
+            float dsv[8];
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+              const int kb = 2 * ks2 + (e >> 2), i = e & 3;
+              float ds = __builtin_amdgcn_exp2f(sacc[kb][qb][i]) * pacc[kb][qb][i];
+              if constexpr (!FULL) {
+                const int j = 16 * kb + 4 * u_m + i;
+                const bool ok = (j <= hi_rel[qb]) & ((j >= lo_rel[qb]) | (j < sink_rel));
+                ds = ok ? ds : 0.f;
+              }
+              dsv[e] = ds;
+            }
+            dsb[ks2][qb] = M::pack(dsv);
+            asm volatile("" : "+v"(dsb[ks2][qb]));
+          }
+      };
+      if (full) {
+        body(std::true_type{});
+      } else {
+        body(std::false_type{});
+      }
+      int t_off = t_row;
+      asm volatile("" : "+v"(t_off));
+#pragma unroll
+      for (int ks2 = 0; ks2 < 2; ks2++)
+#pragma unroll
+        for (int d = 0; d < DB; d++) {
+          const int off = (t_off ^ (d << 5)) + ks2 * 32 * C::ROWB;
+          const V8 kt = tr_pair<V8>(kc + off, kc + off + 16 * C::ROWB);
+#pragma unroll
+          for (int qb = 0; qb < 2; qb++) dq_acc[d][qb] = M::mfma16(kt, dsb[ks2][qb], dq_acc[d][qb]);
+        }
+      {
+        constexpr int NFR = 2 * DB, AH = RSWA_DQ_AH2;  // transposed fragments (2 reads, 2 MFMAs each)
+        __builtin_amdgcn_sched_group_barrier(0x100, 2 * AH, 0);
+#pragma unroll
+        for (int i = 0; i < NFR - AH; i++) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 2 * AH, 0);
+      }
     }
     __syncthreads();
   };
@@ -748,17 +804,17 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(const AttnArgs a) {
   }
 
   // ---- epilogue: dq = scale * acc, transposed through LDS for 16-byte stores ------
+  // element i of dq_acc[d][qb] is dQ[query 16 qb + r][16 d + 4 u + i]
   char* stage = (wave & 3) == 0 ? k_s0 : (wave & 3) == 1 ? k_s1 : (wave & 3) == 2 ? v_s0 : v_s1;
   for (int half = 0; half < 2; half++) {
     if ((wave >> 2) == half) {
 #pragma unroll
-      for (int d = 0; d < C::DBLK; d++)
+      for (int d = 0; d < DB; d++)
 #pragma unroll
-        for (int i4 = 0; i4 < 4; i4++) {
-          const auto h4 =
-              M::pack4(dq_acc[d][4 * i4] * a.scale, dq_acc[d][4 * i4 + 1] * a.scale,
-                       dq_acc[d][4 * i4 + 2] * a.scale, dq_acc[d][4 * i4 + 3] * a.scale);
-          *(typename M::V4*)(stage + l32 * C::O_STRIDE + (d * 32 + 8 * i4 + 4 * g) * 2) = h4;
+        for (int qb = 0; qb < 2; qb++) {
+          const auto h4 = M::pack4(dq_acc[d][qb][0] * a.scale, dq_acc[d][qb][1] * a.scale,
+                                   dq_acc[d][qb][2] * a.scale, dq_acc[d][qb][3] * a.scale);
+          *(typename M::V4*)(stage + (16 * qb + r) * C::O_STRIDE + (16 * d + 4 * u) * 2) = h4;
         }
     }
     __syncthreads();

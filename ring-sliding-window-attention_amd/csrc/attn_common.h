@@ -127,6 +127,9 @@ struct Mma<__bf16> {
   static __device__ __forceinline__ f32x16 mfma32(V8 a, V8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
+  static __device__ __forceinline__ f32x4 mfma16(V8 a, V8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
   // The same instruction as inline assembly with the accumulator kept in vector registers
   // (for accumulators the vector ALU reads next; the builtin's accumulators live in
   // accumulation registers), and a zero-initialising form (early clobber: the destination
@@ -162,6 +165,9 @@ struct Mma<_Float16> {
   using V4 = f16x4;
   static __device__ __forceinline__ f32x16 mfma32(V8 a, V8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4 mfma16(V8 a, V8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
   }
   static __device__ __forceinline__ void mfma32_vec(V8 a, V8 b, f32x16& c) {
     asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
@@ -204,6 +210,29 @@ template <int CH>
 __device__ __forceinline__ int swz(int row, int chunk) {
   return chunk ^ swz_f<CH>(row);
 }
+// The swizzle of the kernels built on 16x16x32 MFMAs (A / B: lane = row or column l % 16,
+// 8 consecutive k at 8 (l / 16); C: lane = column l % 16, rows 4 (l / 16) + i).  Their access
+// patterns: 16 consecutive rows x 4 consecutive chunks (row fragments, 16-byte reads: lane =
+// row l % 16, chunk 4 ks + l / 16) and 16 consecutive rows x 2 consecutive chunks (transposing
+// 8-byte reads: row 4 (l / 16) + (l % 16) / 4).  The functions are GF(2)-linear in the row and
+// were picked by measurement: of all linear maps, run through both patterns on the hardware,
+// these are among those that reach the full LDS rate in both (an obvious candidate, the row's
+// low three bits shifted up by one with bit 3 as the lowest bit, runs the 16-byte pattern at
+// half rate).  They look at the row's low three bits only.
+template <int CH>
+__device__ __forceinline__ int swz16_f(int row) {
+  if constexpr (CH == 16) {
+    return ((row & 1) ? 0xc : 0) ^ ((row & 2) ? 0x8 : 0) ^ ((row & 4) ? 0x2 : 0);
+  } else {
+    static_assert(CH == 8, "rows of 8 or 16 chunks");
+    return ((row & 1) ? 0x6 : 0) ^ ((row & 2) ? 0x7 : 0) ^ ((row & 4) ? 0x2 : 0);
+  }
+}
+template <int CH, bool W16>
+__device__ __forceinline__ int swz_sel(int row) {
+  if constexpr (W16) return swz16_f<CH>(row);
+  else return swz_f<CH>(row);
+}
 
 typedef __attribute__((__vector_size__(8 * sizeof(short)))) short s16x8;
 
@@ -234,7 +263,7 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rows_rsrc(const void* bas
 // land directly in LDS (buffer_load_dwordx4 ... lds: lane L of a wave writes
 // wave_base + 16 L).  The per-lane byte offsets are computed once (init); a tile load is
 // then N instructions with one scalar offset and no vector arithmetic at all.
-template <int D, int ROWS, int THREADS>
+template <int D, int ROWS, int THREADS, bool W16 = false>
 struct TileDma {
   static constexpr int CPR = D / 8;
   static constexpr int RPI = 64 / CPR;  // rows per wave instruction
@@ -252,7 +281,7 @@ struct TileDma {
     const int lane = tid & 63;
     wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int row = wave * RPI + lane / CPR;
-    voff = (int)(row * stride_elems * 2) + (((lane % CPR) ^ swz_f<CPR>(row)) << 4);
+    voff = (int)(row * stride_elems * 2) + (((lane % CPR) ^ swz_sel<CPR, W16>(row)) << 4);
     step_bytes = (int)(NW * RPI * stride_elems * 2);
   }
   // `soff` = byte offset of the tile's first row inside the resource (wave-uniform)
