@@ -36,7 +36,7 @@ struct FwdCfg {
   static_assert(TILE >= 32 * O_STRIDE, "one wave's epilogue staging fits one tile buffer");
 };
 
-template <typename T, int D>
+template <typename T, int D, bool SKIP>
 __global__ __launch_bounds__(512) void attn_fwd_kernel(const AttnArgs a) {
   using C = FwdCfg<D>;
   using M = Mma<T>;
@@ -264,32 +264,55 @@ __global__ __launch_bounds__(512) void attn_fwd_kernel(const AttnArgs a) {
     if (it + 2 < n_tiles) load_k(it + 2, kfree);
     if (it + 1 < n_tiles) load_v(it + 1, vn);
   };
+  // A tile the block visits may hold no key that this wave's 32 rows can see (the block's
+  // key range is as wide as the window plus all its rows): the wave then skips the tile's
+  // work and only keeps the barriers.  With a short window that is a sizeable share: at
+  // window 1000 and 256 rows per block a wave needs 17 of the block's 20 tiles.
+  // (SKIP is chosen by the host for short windows only: with a long window the test costs
+  // more than the rare skipped tile saves.)
+  auto wave_needs = [&](int it) __attribute__((always_inline)) -> bool {
+    if constexpr (!SKIP) return it < n_tiles;
+    const int j0 = tile_of(it) * C::BN;
+    return it < n_tiles && r0 < len_q && j0 <= wb_last.hi &&
+           (j0 + C::BN - 1 >= wb_first.lo || j0 < a.n_sink);
+  };
   auto iter = [&](int it, const char* kn, char* kfree, const char* vc,
                   char* vn) __attribute__((always_inline)) {
+    // without SKIP both are compile-time true: one path, and after the last tile S(t+1) is
+    // computed from stale LDS contents and never used
+    const bool need_cur = SKIP ? wave_needs(it) : true;
+    const bool need_next = SKIP ? wave_needs(it + 1) : true;
     if (late) prefetch(it, kfree, vn);
-    mask(it, s_cur);
     V8 pb[4];
-    const float alpha = softmax(s_cur, pb);
-    rescale(alpha);
+    if (need_cur) {
+      mask(it, s_cur);
+      const float alpha = softmax(s_cur, pb);
+      rescale(alpha);
+    }
     if (!late) wait_dma();
     lds_barrier();
     if (!late) prefetch(it, kfree, vn);
-    // matrix phase as ONE basic block (after the last tile S(t+1) is computed from stale
-    // LDS contents and never used), LDS reads scheduled four fragments ahead of their MFMA
-    pv_acc(vc, pb);
-    qk(kn, s_cur);
-    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+    if (need_cur && need_next) {
+      // matrix phase as ONE basic block, LDS reads scheduled four fragments ahead of their MFMA
+      pv_acc(vc, pb);
+      qk(kn, s_cur);
+      __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
 #pragma unroll
-    for (int i = 0; i < 12; i++) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-    }
+      for (int i = 0; i < 12; i++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      }
 #pragma unroll
-    for (int i = 0; i < 16; i++) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      for (int i = 0; i < 16; i++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+    } else if (need_cur) {
+      pv_acc(vc, pb);
+    } else if (need_next) {
+      qk(kn, s_cur);
     }
-    __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
     if (late) wait_dma();
     lds_barrier();
   };
@@ -301,7 +324,7 @@ __global__ __launch_bounds__(512) void attn_fwd_kernel(const AttnArgs a) {
   if (n_tiles > 1) load_k(1, k_s1);
   __syncthreads();
   if (late) lds_barrier();
-  if (n_tiles > 0) qk(k_s0, s_cur);
+  if (wave_needs(0)) qk(k_s0, s_cur);
   lds_barrier();
   for (int it = 0; it < n_tiles; it += 2) {
     iter(it, k_s1, k_s0, v_s0, v_s1);
@@ -349,10 +372,14 @@ __global__ __launch_bounds__(512) void attn_fwd_kernel(const AttnArgs a) {
 
 // Explicit instantiations: with implicit instantiation alone this hipcc emits the host
 // launch stubs of only some of the four variants.
-template __global__ void attn_fwd_kernel<__bf16, 128>(const AttnArgs);
-template __global__ void attn_fwd_kernel<__bf16, 64>(const AttnArgs);
-template __global__ void attn_fwd_kernel<_Float16, 128>(const AttnArgs);
-template __global__ void attn_fwd_kernel<_Float16, 64>(const AttnArgs);
+#define RSWA_INSTANTIATE(T, D)                                               \
+  template __global__ void attn_fwd_kernel<T, D, false>(const AttnArgs);     \
+  template __global__ void attn_fwd_kernel<T, D, true>(const AttnArgs);
+RSWA_INSTANTIATE(__bf16, 128)
+RSWA_INSTANTIATE(__bf16, 64)
+RSWA_INSTANTIATE(_Float16, 128)
+RSWA_INSTANTIATE(_Float16, 64)
+#undef RSWA_INSTANTIATE
 
 template <typename T, int D>
 int launch_fwd(AttnArgs& a, hipStream_t stream) {
@@ -368,9 +395,18 @@ int launch_fwd(AttnArgs& a, hipStream_t stream) {
     a.n_work = a.n_tile * units * a.batch;
   }
   if (a.n_work == 0) return RSWA_OK;
+  // keys a row sees at most; the per-wave tile skip pays when the rows of a block beyond one
+  // wave's 32 add a tenth or more to that span
+  const int64_t span = (a.wl < 0 || a.wr < 0) ? (int64_t)1 << 40 : (int64_t)a.wl + a.wr + 1;
+  const bool skip = (bm - 32) * 10 >= span + bm;
   clear_launch_error();
-  hipLaunchKernelGGL((attn_fwd_kernel<T, D>), dim3(padded_grid(a.n_work)), dim3(C::THREADS), 0,
-                     stream, a);
+  if (skip) {
+    hipLaunchKernelGGL((attn_fwd_kernel<T, D, true>), dim3(padded_grid(a.n_work)),
+                       dim3(C::THREADS), 0, stream, a);
+  } else {
+    hipLaunchKernelGGL((attn_fwd_kernel<T, D, false>), dim3(padded_grid(a.n_work)),
+                       dim3(C::THREADS), 0, stream, a);
+  }
   return check_launch("attn_fwd");
 }
 
