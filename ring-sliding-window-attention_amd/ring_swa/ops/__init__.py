@@ -1,4 +1,11 @@
-"""Kernel-level operators of the single-GPU path (HIP, gfx950)."""
+"""Kernel-level operators of the attention path (HIP, gfx950) and the operators of the ring
+loops built on them; same names as the upstream package exports from ``ring_swa.ops``."""
+from .accum import (
+    flash_attn_bwd_func,
+    flash_attn_fwd_func,
+    flash_attn_varlen_bwd_func,
+    flash_attn_varlen_fwd_func,
+)
 from .band_attn import (
     attn_bwd,
     attn_fwd,
@@ -8,6 +15,7 @@ from .band_attn import (
     wrapped_flash_attn_fwd_varlen,
 )
 from .lse_merge import merge_attn_out
+from .p2p import get_group_local_to_global_rank_map, ring_attn_p2p_communicate
 
 __all__ = [
     "attn_fwd",
@@ -16,5 +24,11 @@ __all__ = [
     "wrapped_flash_attn_fwd_varlen",
     "wrapped_flash_attn_bwd",
     "wrapped_flash_attn_bwd_varlen",
+    "flash_attn_fwd_func",
+    "flash_attn_bwd_func",
+    "flash_attn_varlen_fwd_func",
+    "flash_attn_varlen_bwd_func",
     "merge_attn_out",
+    "ring_attn_p2p_communicate",
+    "get_group_local_to_global_rank_map",
 ]

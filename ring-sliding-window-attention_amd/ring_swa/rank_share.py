@@ -20,6 +20,8 @@ from typing import List, Optional, Sequence, Tuple
 
 import torch
 
+from .ops.accum import (flash_attn_bwd_func, flash_attn_fwd_func, flash_attn_varlen_bwd_func,
+                        flash_attn_varlen_fwd_func)
 from .ops.band_attn import attn_bwd, attn_fwd, bwd_workspace_bytes
 from .ops.lse_merge import merge_attn_out
 
@@ -184,9 +186,36 @@ def _join(side: "torch.cuda.Stream", device: torch.device) -> None:
     torch.cuda.current_stream(device).wait_stream(side)
 
 
+def _forward_blocks_accum(q, k, v, prev_kv, plan, scale, local_cu):
+    """The blocks through the accumulating block operators, upstream's flow and accumulator
+    types (``ring_swa/sliding_window/nonvarlen.py:53-59, 95-154``): fp32 output and fp64 LSE
+    start from the merge identity, every block is merged into its row range, one cast at the
+    end."""
+    b, s, hq, _ = q.shape
+    out = torch.zeros_like(q, dtype=torch.float32)
+    lse = torch.full((b, hq, s), float("-inf"), dtype=torch.float64, device=q.device)
+    for (i, qs, ks, window, causal) in plan:
+        if i == 0:
+            kv = torch.stack([k, v])
+            if local_cu is not None:
+                flash_attn_varlen_fwd_func(q, kv, scale, window, local_cu, local_cu, None, None,
+                                           causal, out, lse)
+            else:
+                flash_attn_fwd_func(q, kv, scale, window, causal, out, lse)
+        else:
+            flash_attn_fwd_func(q[:, qs], prev_kv[i - 1][:, :, ks], scale, window, causal,
+                                out[:, qs], lse[:, :, qs])
+    return out.to(q.dtype), lse.float()
+
+
 def _forward_blocks(q, k, v, prev_kv, plan, scale, local_cu, ring_dtypes):
     """Run the planned blocks and merge them.  Dense 4-d tensors (batch 1 when packed)."""
     assert plan and plan[0][0] == 0, "the diagonal block comes first: it covers every row"
+    if ring_dtypes or len(plan) > 2:
+        # With two blocks the 16-bit running output is merged once and rounded once, the same
+        # bits as the fp32 accumulator gives; from three blocks on every further merge would
+        # add a rounding the reference does not have, so its accumulators are used.
+        return _forward_blocks_accum(q, k, v, prev_kv, plan, scale, local_cu)
     side = _fork(q.device) if len(plan) > 1 else None
     caller = torch.cuda.current_stream(q.device)
     parts = []
@@ -208,12 +237,6 @@ def _forward_blocks(q, k, v, prev_kv, plan, scale, local_cu, ring_dtypes):
     if side is not None:
         _join(side, q.device)
     _, out, lse = parts[0]
-    if ring_dtypes or len(parts) > 2:
-        # accumulator types of ring_swa/sliding_window/nonvarlen.py:53-59.  With two blocks
-        # the 16-bit running output is merged once and rounded once, the same bits as the
-        # fp32 accumulator gives; from three blocks on every further merge would add a
-        # rounding the reference does not have, so the fp32 / fp64 pair is used regardless.
-        out, lse = out.float(), lse.double()
     for qs, o_i, l_i in parts[1:]:
         merge_attn_out(out[:, qs], lse[:, :, qs], o_i, l_i)
     return out.to(q.dtype), lse.float()
@@ -225,37 +248,33 @@ def _backward_blocks(q, k, v, prev_kv, out, lse, do, plan, scale, local_cu):
     assert plan and plan[0][0] == 0
     if len(plan) == 2:
         return _backward_two_blocks(q, k, v, prev_kv, out, lse, do, plan, scale, local_cu)
-    single = len(plan) == 1
-    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    # one block, or three and more: the accumulating flow of upstream's backward
+    # (ring_swa/sliding_window/nonvarlen.py:203-206, 233-321) on the block operators; dq and
+    # the own chunk's dkv are summed in fp32, the previous chunks' gradients are what a ring
+    # would send back
+    if len(plan) == 1:
+        dq, dkv = torch.empty_like(q), torch.empty_like(torch.stack([k, v]))
+    else:
+        dq = torch.zeros_like(q, dtype=torch.float32)
+        dkv = torch.empty_like(torch.stack([k, v]))
     dprev = [torch.zeros_like(kv) for kv in prev_kv]
-    # every buffer is allocated on the caller's stream before the fork
-    dq_parts = [(qs, torch.empty_like(q[:, qs])) for (i, qs, _, _, _) in plan if i > 0]
-    side = None if single else _fork(q.device)
-    n = 0
     for (i, qs, ks, window, causal) in plan:
         if i == 0:
+            kv = torch.stack([k, v])
+            dq_0 = dq if len(plan) == 1 else torch.empty_like(q)
             if local_cu is not None:
-                attn_bwd(q[0], k[0], v[0], out[0], lse[0], do[0], dq[0], dk[0], dv[0], scale,
-                         window, causal, local_cu, local_cu)
+                flash_attn_varlen_bwd_func(q, kv, out, lse, do, dq_0, dkv, local_cu, local_cu,
+                                           None, None, scale, window, causal)
             else:
-                attn_bwd(q, k, v, out, lse, do, dq, dk, dv, scale, window, causal)
+                flash_attn_bwd_func(q, kv, out, lse, do, dq_0, dkv, scale, window, causal)
+            if len(plan) > 1:
+                dq += dq_0
         else:
-            # rows / keys outside the slices receive nothing from this block
-            kk, vv = prev_kv[i - 1][0], prev_kv[i - 1][1]
-            dkv = dprev[i - 1]
-            with torch.cuda.stream(side):
-                attn_bwd(q[:, qs], kk[:, ks], vv[:, ks], out[:, qs], lse[:, :, qs], do[:, qs],
-                         dq_parts[n][1], dkv[0][:, ks], dkv[1][:, ks], scale, window, causal)
-            n += 1
-    if not single:
-        _join(side, q.device)
-        # dq accumulates in fp32 across the blocks, as upstream does
-        # (ring_swa/sliding_window/nonvarlen.py:203, 318-321)
-        dq_acc = dq.float()
-        for qs, dq_i in dq_parts:
-            dq_acc[:, qs].add_(dq_i)
-        dq = dq_acc.to(q.dtype)
-    return (dq, dk, dv, *dprev)
+            dq_i = torch.empty_like(q[:, qs])
+            flash_attn_bwd_func(q[:, qs], prev_kv[i - 1][:, :, ks], out[:, qs], lse[:, :, qs],
+                                do[:, qs], dq_i, dprev[i - 1][:, :, ks], scale, window, causal)
+            dq[:, qs] += dq_i
+    return (dq.to(q.dtype), dkv[0], dkv[1], *dprev)
 
 
 def _backward_two_blocks(q, k, v, prev_kv, out, lse, do, plan, scale, local_cu):

@@ -3,8 +3,8 @@
 Same names, positional order and argument meaning as the upstream package
 (``ring_swa/sliding_window/nonvarlen.py:341-408`` and
 ``ring_swa/sliding_window/varlen.py:362-441``).  With ``cp_group=None`` the call
-runs the HIP band-attention kernels directly; the multi-GPU ring
-(``cp_group`` given) is not part of this build and raises.
+runs the HIP band-attention kernels directly; with a ``cp_group`` it goes through
+``ring_swa/ring.py`` (one process per GPU, chunks exchanged over ``torch.distributed``).
 """
 from __future__ import annotations
 
@@ -45,12 +45,25 @@ class BandAttnFunc(torch.autograd.Function):
         return dq, dk, dv, None, None, None, None
 
 
-def _reject_ring(cp_group):
-    if cp_group is not None:
-        raise NotImplementedError(
-            "this build covers the single-GPU path (cp_group=None) and one rank's share of the "
-            "ring (ring_swa.rank_share); the multi-GPU ring itself is not implemented"
+def _ring_ranks(cp_group, cp_size, cp_local_rank, cp_prev_global_rank, cp_next_global_rank):
+    """The rank arguments of a call with ``cp_group``: ``cp_size`` and ``cp_local_rank`` default
+    to the group's own, and the neighbours' global ranks, if given, must be the ones the
+    group's rank map yields (``README.md:63-64`` of the upstream package obtains them from it)."""
+    import torch.distributed as dist
+
+    from .ops.p2p import get_group_local_to_global_rank_map
+
+    if cp_size is None:
+        cp_size = dist.get_world_size(cp_group)
+    if cp_local_rank is None:
+        cp_local_rank = dist.get_rank(cp_group)
+    gmap = get_group_local_to_global_rank_map(cp_group)
+    for given, other in ((cp_prev_global_rank, (cp_local_rank - 1) % cp_size),
+                         (cp_next_global_rank, (cp_local_rank + 1) % cp_size)):
+        assert given is None or given == gmap[other], (
+            f"neighbour rank {given} is not the group's rank {other} (global {gmap[other]})"
         )
+    return int(cp_size), int(cp_local_rank)
 
 
 def _check_dense(q, k, v):
@@ -73,7 +86,7 @@ def _check_packed(q, k, v, cu_seqlens, cp_size):
     # cp_size means 1 on the single-GPU path and the check is done without touching the
     # device: the packed tensors must hold cu_seqlens[-1] rows, which the kernel bounds
     # by q.shape[0] anyway.
-    assert cp_size in (None, 1), "cp_size > 1 needs cp_group (not part of this build)"
+    assert cp_size in (None, 1), "cp_size > 1 needs cp_group"
 
 
 def ring_sliding_window_attn(
@@ -94,8 +107,13 @@ def ring_sliding_window_attn(
     ``window_size=(w, 0), causal=True`` (``ring_swa/sliding_window/nonvarlen.py:376-386``).
     Returns the attention output, same shape and dtype as ``q``.
     """
-    _reject_ring(cp_group)
     _check_dense(q, k, v)
+    if cp_group is not None:
+        from .ring import ring_attn
+
+        cp_size, cp_local_rank = _ring_ranks(cp_group, cp_size, cp_local_rank,
+                                             cp_prev_global_rank, cp_next_global_rank)
+        return ring_attn(q, k, v, window_size, cp_group, cp_size, cp_local_rank, softmax_scale)
     return BandAttnFunc.apply(q, k, v, int(window_size), softmax_scale, None, 0)
 
 
@@ -117,6 +135,13 @@ def ring_sliding_window_attn_varlen(
     ``ring_swa/sliding_window/varlen.py:401-417``.  No host synchronisation: the
     longest sequence length is never read back.
     """
-    _reject_ring(cp_group)
+    if cp_group is not None:
+        from .ring import ring_attn
+
+        _check_packed(q, k, v, cu_seqlens, 1)
+        cp_size, cp_local_rank = _ring_ranks(cp_group, cp_size, cp_local_rank,
+                                             cp_prev_global_rank, cp_next_global_rank)
+        return ring_attn(q, k, v, window_size, cp_group, cp_size, cp_local_rank, softmax_scale,
+                         cu_seqlens)
     _check_packed(q, k, v, cu_seqlens, cp_size)
     return BandAttnFunc.apply(q, k, v, int(window_size), softmax_scale, cu_seqlens.contiguous(), 0)

@@ -33,7 +33,16 @@ import torch
 
 from .ops.band_attn import attn_bwd, attn_fwd
 from .ops.lse_merge import merge_attn_out
-from .sliding_window import BandAttnFunc, _check_dense, _check_packed, _reject_ring
+from .sliding_window import BandAttnFunc, _check_dense, _check_packed
+
+
+def _reject_ring(cp_group):
+    if cp_group is not None:
+        raise NotImplementedError(
+            "streaming-LLM attention over a context-parallel group (sink broadcast, sink-gradient "
+            "reduction) is not part of this build; sliding-window attention is "
+            "(ring_swa.ring_sliding_window_attn[_varlen] with cp_group)"
+        )
 
 
 class SinkWindowSplitFunc(torch.autograd.Function):
