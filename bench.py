@@ -59,10 +59,11 @@ def event_ms(fn, n, warm=3):
 def cpu_baseline(seconds_budget: float = 25.0):
     """The oracle (PyTorch masked softmax, fp32, autograd) on the host cores.
 
-    Bounded sample of the headline workload: same structure scaled down — chunk 4096
-    with a 4096-token predecessor, window 2048, 4 q / 1 kv heads, head_dim 128 — plus
-    the reference's own CPU-runnable case (fp32, seq 1024, 4 heads, head_dim 64,
-    window 256, seed 0)."""
+    ``value`` = the reference's own CPU-runnable case (fp32, batch 1, seq 1024, 4 q = 4 kv
+    heads, head_dim 64, window 256, seed 0, scale 1/8, dO ~ N(0,1)): 2 warm-up + 5 timed
+    forward+backward passes, median, converted with that case's 0.83 GFLOP.  Beside it a
+    bounded sample of the headline workload's structure scaled down (4096 queries against
+    8192 keys = own + previous chunk, window 2048, 4 q / 1 kv heads, head_dim 128)."""
     import torch
 
     from oracle import attention_oracle as O
@@ -70,42 +71,76 @@ def cpu_baseline(seconds_budget: float = 25.0):
     cores = os.cpu_count() or 1
     torch.set_num_threads(cores)
 
-    def run(sq, sk, hq, hk, d, w, seed):
-        g = torch.Generator().manual_seed(seed)
-        q = torch.randn(1, sq, hq, d, generator=g)
-        k = torch.randn(1, sk, hk, d, generator=g)
-        v = torch.randn(1, sk, hk, d, generator=g)
-        do = torch.randn(1, sq, hq, d, generator=g)
+    def run(sq, sk, hq, hk, d, w, seed, warm, n_max, budget):
+        torch.manual_seed(seed)
+        q = torch.randn(1, sq, hq, d)
+        k = torch.randn(1, sk, hk, d)
+        v = torch.randn(1, sk, hk, d)
+        do = torch.randn(1, sq, hq, d)
         fn = lambda: O.attention_fwd_bwd(  # noqa: E731
             lambda q, k, v: O.window_attention(q, k, v, d ** -0.5, (w, 0), True), q, k, v, do)
-        fn()
+        for _ in range(warm):
+            fn()
         ts = []
         t_start = time.perf_counter()
-        while len(ts) < 5 and (time.perf_counter() - t_start < seconds_budget / 2 or len(ts) < 2):
+        while len(ts) < n_max and (time.perf_counter() - t_start < budget or len(ts) < 2):
             t0 = time.perf_counter()
             fn()
             ts.append(time.perf_counter() - t0)
         ts.sort()
-        return ts[len(ts) // 2]
+        return ts[len(ts) // 2], len(ts)
 
+    t1, n1 = run(1024, 1024, 4, 4, 64, 256, 0, 2, 5, seconds_budget / 2)
+    c1_flops = 14 * 64 * band_pairs(1024, 256) * 4
     # sample of the rank share: queries = last 4096 positions of 8192 keys, window 2048
     sq, sk, hq, hk, d, w = 4096, 8192, 4, 1, 128, 2048
-    t = run(sq, sk, hq, hk, d, w, 0)
+    t, n = run(sq, sk, hq, hk, d, w, 0, 1, 5, seconds_budget / 2)
     pairs = sq * (w + 1)  # every query has a full window inside the two chunks
-    sample_tflops = 14 * d * pairs * hq / t / 1e12
-    t1 = run(1024, 1024, 4, 4, 64, 256, 0)
-    c1_gflops = 14 * 64 * band_pairs(1024, 256) * 4 / t1 / 1e9
     return {
-        "value": sample_tflops,
+        "value": c1_flops / t1 / 1e12,
         "unit": "TFLOP/s",
         "cores": cores,
         "threads": torch.get_num_threads(),
         "kind": "port",
-        "sample": "oracle fp32 fwd+bwd (autograd) of a scaled-down rank share: 4096 queries x "
-                  "8192 keys (own + previous chunk), window 2048, 4 q / 1 kv heads, head_dim 128; "
-                  f"median {t * 1e3:.1f} ms",
-        "c1_fp32_seq1024_h4_d64_w256": {"ms": t1 * 1e3, "GFLOP/s": c1_gflops},
+        "sample": "oracle fp32 fwd+bwd (autograd) of the CPU case: batch 1, seq 1024, 4 q = 4 kv "
+                  f"heads, head_dim 64, window 256, seed 0; median of {n1} passes {t1 * 1e3:.1f} ms "
+                  f"= {c1_flops / t1 / 1e9:.1f} GFLOP/s",
+        "c1_ms": t1 * 1e3,
+        "scaled_down_rank_share": {
+            "TFLOP/s": 14 * d * pairs * hq / t / 1e12, "ms": t * 1e3, "passes": n,
+            "what": "4096 queries x 8192 keys (own + previous chunk), window 2048, 4 q / 1 kv "
+                    "heads, head_dim 128, fp32"},
     }
+
+
+def log_uniform_lengths(total, lo, hi, seed):
+    """Sequence lengths drawn log-uniform in [lo, hi] until they cover ``total``, the last one
+    truncated (the generator of the packed configuration)."""
+    import math
+
+    import torch
+
+    g = torch.Generator().manual_seed(seed)
+    lens = []
+    while sum(lens) < total:
+        x = math.exp(math.log(lo) + torch.rand(1, generator=g).item() * (math.log(hi) - math.log(lo)))
+        lens.append(int(x))
+    lens[-1] -= sum(lens) - total
+    if lens[-1] == 0:
+        lens.pop()
+    return lens
+
+
+def global_pairs_of_rows(cu, w, row0, row1, n_sink=0):
+    """Visible (query, key) pairs of the packed rows [row0, row1): every row sees
+    min(position in its sequence, w) + 1 keys, plus the sinks that lie before its window."""
+    total = 0
+    for a, b in zip(cu[:-1], cu[1:]):
+        lo, hi = max(a, row0), min(b, row1)
+        for p in range(lo, hi):
+            pos = p - a
+            total += min(pos, w) + 1 + max(0, min(n_sink, pos - w))
+    return total
 
 
 def main():
@@ -203,11 +238,32 @@ def main():
             "workload": "c3_rank_share",
             "detail": "1 rank of virtual cp 8: chunk 8192 of seq 65536, 32 q / 8 kv heads, "
                       "head_dim 128, window 4096; own-chunk band + previous-chunk corner + LSE "
-                      "merge; fwd+bwd via autograd",
+                      "merge; fwd+bwd via autograd; ring_dtypes=False: the two blocks' 16-bit outputs and fp32 LSE "
+                      "are merged once; the reference's accumulator types (fp32 output, fp64 "
+                      "LSE, one merge per block) are ring_dtypes=True, timed as "
+                      "ms_per_step_ring_dtypes",
+            "ring_dtypes": False,
             "batch": 1, "chunk": S, "heads_q": HQ, "heads_kv": HK, "head_dim": D, "window": W,
             "pairs_per_head": pairs, "flops_per_step": flops,
         },
     }
+
+    # the same step with the reference's accumulator types (fp32 output, fp64 LSE, merged
+    # through the block operators; two cast passes)
+    def step_ring_dtypes():
+        for t in (q, k, v, prev):
+            t.grad = None
+        out = ring_swa.ring_rank_share_attn(q, k, v, [prev], W, CP, RANK, ring_dtypes=True)
+        out.backward(do)
+
+    for _ in range(3):
+        step_ring_dtypes()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step_ring_dtypes()
+    torch.cuda.synchronize()
+    rec["ms_per_step_ring_dtypes"] = (time.perf_counter() - t0) * 1e3 / args.steps
 
     # ---- roofline of the dominant kernel: backward dK/dV kernel, own-chunk block ----
     # Algorithmic FLOPs per visible (query, key) pair and q head: forward 4 D (S, PV);
@@ -291,6 +347,98 @@ def main():
                 "fwd_ms": f2, "bwd_ms": b2, "TFLOP/s": 14 * 128 * p2 / (f2 + b2) / 1e9,
                 "pct_bf16_mfma_peak": 14 * 128 * p2 / (f2 + b2) / 1e9 / PEAK_BF16_TFLOPS * 100}
             del q2, k2, v2, do2, o2, l2, g2
+            # config 4: packed pack of 32768 tokens (log-uniform lengths), window 2048; one rank
+            # slice of virtual cp 4 whose chunk starts inside a sequence (diagonal packed block +
+            # rectangle on the previous chunk + merge), and the whole pack in one call
+            import itertools
+
+            T4, CP4, W4 = 32768, 4, 2048
+            lens4 = log_uniform_lengths(T4, 64, 16384, seed=0)
+            cu4 = [0] + list(itertools.accumulate(lens4))
+            s4 = T4 // CP4
+            r4 = next(r for r in range(1, CP4) if (r * s4) not in cu4)
+            q4, do4 = mk(T4, HQ, D), mk(T4, HQ, D)
+            k4, v4 = mk(T4, HK, D), mk(T4, HK, D)
+            sl = slice(r4 * s4, (r4 + 1) * s4)
+            ps = slice((r4 - 1) * s4, r4 * s4)
+            qr, kr, vr = (t[sl].clone().requires_grad_() for t in (q4, k4, v4))
+            pr = torch.stack([k4[ps], v4[ps]]).requires_grad_()
+
+            @torch.enable_grad()
+            def c4_slice():
+                for t in (qr, kr, vr, pr):
+                    t.grad = None
+                ring_swa.ring_rank_share_attn_varlen(qr, kr, vr, [pr], W4, cu4, CP4, r4).backward(do4[sl])
+
+            cu4_dev = torch.tensor(cu4, dtype=torch.int32, device=dev)
+            qg4, kg4, vg4 = (t.clone().requires_grad_() for t in (q4, k4, v4))
+
+            @torch.enable_grad()
+            def c4_whole():
+                for t in (qg4, kg4, vg4):
+                    t.grad = None
+                ring_swa.ring_sliding_window_attn_varlen(qg4, kg4, vg4, W4, cu4_dev, cp_size=1).backward(do4)
+
+            t_slice, _ = event_ms(c4_slice, 10)
+            t_whole, _ = event_ms(c4_whole, 10)
+            p_slice = global_pairs_of_rows(cu4, W4, r4 * s4, (r4 + 1) * s4)
+            p_whole = sum(band_pairs(l, W4) for l in lens4)
+            rec["c4_varlen_t32768_w2048"] = {
+                "sequences": len(lens4), "rank": r4,
+                "rank_slice": {"ms": t_slice, "pairs_per_head": p_slice,
+                               "TFLOP/s": tf(14 * D * p_slice * HQ, t_slice),
+                               "pct_bf16_mfma_peak": tf(14 * D * p_slice * HQ, t_slice) / PEAK_BF16_TFLOPS * 100},
+                "whole_pack_one_call": {"ms": t_whole, "pairs_per_head": p_whole,
+                                        "TFLOP/s": tf(14 * D * p_whole * HQ, t_whole),
+                                        "pct_bf16_mfma_peak": tf(14 * D * p_whole * HQ, t_whole) / PEAK_BF16_TFLOPS * 100}}
+            del q4, k4, v4, do4, qr, kr, vr, pr, qg4, kg4, vg4
+            # config 5: packed streaming-LLM, 65536 tokens in 4 sequences (cut points not
+            # multiples of the kernels' tiles), sinks + window 4092, sink keys x4
+            T5, W5 = 65536, 4092
+            g5 = torch.Generator().manual_seed(0)
+            cuts = sorted((torch.randperm(T5 // 1024 - 1, generator=g5)[:3] + 1).tolist())
+            cu5 = [0] + [c * 1024 + 37 + 64 * i for i, c in enumerate(cuts)] + [T5]
+            lens5 = [b - a for a, b in zip(cu5[:-1], cu5[1:])]
+            cu5_dev = torch.tensor(cu5, dtype=torch.int32, device=dev)
+            q5, do5 = mk(T5, HQ, D), mk(T5, HQ, D)
+            k5, v5 = mk(T5, HK, D), mk(T5, HK, D)
+            c5 = {"lengths": lens5}
+            for n_sink in (1, 4):
+                kk5 = k5.clone()
+                for c in cu5[:-1]:
+                    kk5[c:c + n_sink] *= 4
+                pairs5 = global_pairs_of_rows(cu5, W5, 0, T5, n_sink) if n_sink == 4 else \
+                    sum(band_pairs(l, W5) + max(0, l - 1 - W5) for l in lens5)
+                for impl in ("fused", "split"):
+                    qg, kg, vg = (t.clone().requires_grad_() for t in (q5, kk5, v5))
+                    kw = {} if n_sink == 1 else {"num_sink_tokens": n_sink}
+
+                    @torch.enable_grad()
+                    def c5_step():
+                        for t in (qg, kg, vg):
+                            t.grad = None
+                        ring_swa.ring_streaming_llm_attn_varlen(qg, kg, vg, W5, cu5_dev, cp_size=1,
+                                                                impl=impl, **kw).backward(do5)
+
+                    t5, _ = event_ms(c5_step, 5, warm=2)
+                    c5[f"{impl}_sinks{n_sink}"] = {
+                        "ms": t5, "pairs_per_head": pairs5, "TFLOP/s": tf(14 * D * pairs5 * HQ, t5),
+                        "pct_bf16_mfma_peak": tf(14 * D * pairs5 * HQ, t5) / PEAK_BF16_TFLOPS * 100}
+                    del qg, kg, vg
+            rec["c5_slm_varlen_t65536_w4092"] = c5
+            del q5, k5, v5, do5, kk5
+            # the merge of that configuration's split path: all tokens x 32 heads, 16-bit
+            # outputs and fp32 LSE on both sides (780 bytes per row)
+            acc = torch.randn(1, T5, HQ, D, device=dev).bfloat16()
+            lacc = torch.randn(1, HQ, T5, device=dev)
+            new = torch.randn(1, T5, HQ, D, device=dev).bfloat16()
+            lnew = torch.randn(1, HQ, T5, device=dev)
+            med, avg = event_ms(lambda: merge_attn_out(acc, lacc, new, lnew), 20)
+            nbytes = T5 * HQ * (6 * D + 12)
+            merge_c5 = {"rows": T5 * HQ, "bytes": nbytes, "us": med * 1e3, "GB/s": nbytes / med / 1e6,
+                        "pct_hbm_peak": nbytes / med / 1e6 / PEAK_HBM_GBPS * 100,
+                        "dtypes": "o bf16, new o bf16, lse fp32, new lse fp32"}
+            del acc, lacc, new, lnew
             # merge kernel: rank-share shape (rows [:4096] x 32 heads) and the sweep's top point
             merges = {}
             for name, rows_s in (("c3_rows4096", 4096), ("sweep_s131072", 131072)):
@@ -323,6 +471,7 @@ def main():
                                        "GB/s": rows_s * HQ * (10 * D + 20) / med / 1e6}
                 del acc, lacc, new, lnew
             merges["sweep_ring_dtypes"] = sweep
+            merges["c5_rows65536_naive_dtypes"] = merge_c5
             rec["merge"] = merges
             rec["merge_GBps"] = merges["sweep_s131072"]["GB/s"]
 
