@@ -161,8 +161,16 @@ typedef struct rswa_attn_params {
    * accumulator over two ring blocks gives, ring_swa/sliding_window/nonvarlen.py:318-321,
    * without the extra passes over dq).  dk / dv are always overwritten. */
   int32_t dq_accumulate;
-  int32_t reserved_;
+  /* RSWA_ADDR_AUTO (0): tiles are fetched through 32-bit offsets that count from a sequence's
+   * first row when every sequence of q, k, v (and dout) spans less than 2 GiB (rows x row
+   * stride), from each tile's first row otherwise -- a sequence may then span anything, only
+   * one row stride must stay below 8 MiB.  RSWA_ADDR_FAR (1) selects the second form whatever
+   * the sizes (same results; a few per cent slower). */
+  int32_t addressing;
 } rswa_attn_params;
+
+#define RSWA_ADDR_AUTO 0
+#define RSWA_ADDR_FAR 1
 
 int rswa_attn_fwd(const rswa_attn_params* p, void* stream);
 int rswa_attn_bwd(const rswa_attn_params* p, void* stream);
@@ -186,9 +194,10 @@ int rswa_attn_bwd_phases(const rswa_attn_params* p, void* stream, int phases);
  * (every GPU the library runs on holds it until the process ends); p->workspace and
  * p->workspace_bytes are ignored.  No counterpart in the upstream package: it is for
  * callers that cannot allocate device memory around the call - code under HIP graph
- * capture, tight serving loops, harnesses that forbid hipMalloc.  Shapes whose
- * rswa_attn_bwd_workspace_bytes() exceed the buffer (more than 4 194 304 (row, q head)
- * pairs) are refused with RSWA_ERR_UNSUPPORTED.  The buffer's address is looked up on the
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  Shapes whose statistics
+ * (8 bytes per (row, q head) pair) exceed the buffer -- more than 4 194 304 pairs -- are
+ * refused with RSWA_ERR_UNSUPPORTED; the dK/dV kernel runs one block per key tile here,
+ * whatever the shape (no partial sums).  The buffer's address is looked up on the
  * first call on each device (the device must be current, as for every other call); nothing
  * in it has to be cleared between calls, the statistics kernel rewrites what the others
  * read.  All calls on one GPU share the one buffer: calls that may overlap in time on the
@@ -197,8 +206,12 @@ int rswa_attn_bwd_phases(const rswa_attn_params* p, void* stream, int phases);
 #define RSWA_BWD_STATIC_MAX_BYTES (32u << 20)
 int rswa_attn_bwd_static(const rswa_attn_params* p, void* stream);
 
-/* Scratch rswa_attn_bwd needs for these shapes: two fp32 values per (row, q head) —
- * the row sum of dout * out and the LSE in base-2 units. */
+/* Scratch rswa_attn_bwd needs for these shapes: two fp32 values per (row, q head) -- the
+ * row sum of dout * out and the LSE in base-2 units -- and, for launches with so few key
+ * tiles (fewer than 129 blocks of 256 keys x kv head) that the q heads of each GQA group are
+ * dealt to 2-4 blocks per tile, one arrival counter per tile and the fp32 partial dK / dV of
+ * every part (256 keys x head_dim x 2 x 4 bytes each).  The call leaves the counters at zero;
+ * nothing in the workspace has to be initialised by the caller. */
 uint64_t rswa_attn_bwd_workspace_bytes(const rswa_attn_params* p);
 
 /* Message of the calling thread's last failed call ("" if none). */

@@ -80,14 +80,21 @@ int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a, bool allow_
                RSWA_ERR_UNSUPPORTED, "attn: q/k/v/out rows must start 16-byte aligned");
   RSWA_REQUIRE(((uintptr_t)p->lse) % 4 == 0, RSWA_ERR_UNSUPPORTED, "attn: lse misaligned");
   {
-    // tiles are fetched through 32-bit buffer offsets relative to a (sequence, head) slice
-    const int64_t rq = packed ? p->total_q : p->seqlen_q, rk = packed ? p->total_k : p->seqlen_k;
+    // Tiles are fetched through 32-bit byte offsets.  The rows of one tile (at most
+    // kMaxTileRows) must span less than 2 GiB; when a whole sequence does too, offsets count
+    // from the sequence's first row, otherwise from each tile's (FAR kernels).
     const int64_t lim = (1ll << 31) - 65536;
-    RSWA_REQUIRE(rq * p->q_stride[1] * 2 < lim && rk * p->k_stride[1] * 2 < lim &&
-                     rk * p->v_stride[1] * 2 < lim && p->q_stride[1] >= 0 &&
-                     p->k_stride[1] >= 0 && p->v_stride[1] >= 0,
+    RSWA_REQUIRE(p->q_stride[1] >= 0 && p->k_stride[1] >= 0 && p->v_stride[1] >= 0 &&
+                     p->q_stride[1] * 2 < lim / kMaxTileRows && p->k_stride[1] * 2 < lim / kMaxTileRows &&
+                     p->v_stride[1] * 2 < lim / kMaxTileRows,
                  RSWA_ERR_UNSUPPORTED,
-                 "attn: one sequence of q, k or v spans 2 GiB or more (rows * row stride)");
+                 "attn: row stride of q, k or v is negative or %lld bytes or more",
+                 (long long)(lim / kMaxTileRows));
+    // packed: judged on the whole pack (no sequence is longer)
+    const int64_t rq = packed ? p->total_q : p->seqlen_q, rk = packed ? p->total_k : p->seqlen_k;
+    a.far = (p->addressing == RSWA_ADDR_FAR) || rq * p->q_stride[1] * 2 >= lim ||
+            rk * p->k_stride[1] * 2 >= lim || rk * p->v_stride[1] * 2 >= lim ||
+            (backward && rq * p->dout_stride[1] * 2 >= lim);
   }
 
   a.q = p->q;
@@ -167,11 +174,8 @@ int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a, bool allow_
     RSWA_REQUIRE(rows_aligned(p->dout, p->dout_stride) && rows_aligned(p->dq, p->dq_stride) &&
                      rows_aligned(p->dk, p->dk_stride) && rows_aligned(p->dv, p->dv_stride),
                  RSWA_ERR_UNSUPPORTED, "attn_bwd: dout/dq/dk/dv rows must start 16-byte aligned");
-    {
-      const int64_t rq = packed ? p->total_q : p->seqlen_q;
-      RSWA_REQUIRE(rq * p->dout_stride[1] * 2 < (1ll << 31) - 65536 && p->dout_stride[1] >= 0,
-                   RSWA_ERR_UNSUPPORTED, "attn_bwd: one sequence of dout spans 2 GiB or more");
-    }
+    RSWA_REQUIRE(p->dout_stride[1] >= 0 && p->dout_stride[1] * 2 < ((1ll << 31) - 65536) / kMaxTileRows,
+                 RSWA_ERR_UNSUPPORTED, "attn_bwd: row stride of dout is negative or too large");
     const BwdLayout L = bwd_layout(p, allow_split);
     const uint64_t need = L.total_bytes;
     RSWA_REQUIRE(p->workspace != nullptr || need == 0, RSWA_ERR_INVALID,
@@ -187,8 +191,11 @@ int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a, bool allow_
     a.n_count = L.n_count;
     a.dkv_count = (int32_t*)((char*)p->workspace + L.count_off);
     a.dkv_part = (float*)((char*)p->workspace + L.part_off);
-    RSWA_REQUIRE(2 * delta_bytes(p) < (1ull << 31), RSWA_ERR_UNSUPPORTED,
-                 "attn_bwd: rows * heads_q too large for the statistics workspace");
+    // one load reaches from a row's lse2 to its delta, one array further on
+    RSWA_REQUIRE(delta_bytes(p) < (1ull << 31) - 65536, RSWA_ERR_UNSUPPORTED,
+                 "attn_bwd: rows * heads_q = %lld: each statistics array must stay below 2 GiB "
+                 "(536 854 528 (row, q head) pairs)",
+                 (long long)(delta_bytes(p) / 4));
   }
   return RSWA_OK;
 }

@@ -66,7 +66,7 @@ struct DkvCfg {
   static constexpr int V_TILE = BN * ROWB;
 };
 
-template <typename T, int D, bool SPLIT>
+template <typename T, int D, bool SPLIT, bool FAR>
 __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   using C = DkvCfg<D>;
   using M = Mma<T>;
@@ -180,23 +180,20 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   do_dma.init(a.do_st[1], tid);
   const T* q_base = (const T*)a.q + b * a.q_st[0] + s.q_row0 * a.q_st[1];
   const T* do_base = (const T*)a.dout + b * a.do_st[0] + s.q_row0 * a.do_st[1];
+  // statistics: one load covers both workspace arrays (lse2, then delta `stat_elems` further
+  // on) through a resource based at the tile's first row; rows past the sequence end read a
+  // neighbour's finite values, which the row mask / zero Q, dO rows void
+  // (element counts below 2^30: the host refuses larger statistics arrays)
+  const int stat_elems = (int)(a.delta - a.lse2);  // elements between the two arrays
+  const int stat_end = stat_elems + a.heads_q * (int)a.rows_q;  // end of delta
   const int q_row_bytes = (int)(a.q_st[1] * 2), do_row_bytes = (int)(a.do_st[1] * 2);
-  // bytes from a head's first row to the end of its last row (see make_rows_rsrc)
-  const int q_extent = (len_q - 1) * q_row_bytes + C::ROWB;
-  const int do_extent = (len_q - 1) * do_row_bytes + C::ROWB;
-  // statistics: one resource over both workspace arrays (lse2 then delta); rows past the
-  // sequence end read a neighbour's finite values, which the row mask / zero Q, dO rows void
-  const int64_t stat_elems = a.delta - a.lse2;  // elements between the two arrays
-  const __amdgpu_buffer_rsrc_t st_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)a.lse2, 0, (int)((stat_elems + a.heads_q * a.rows_q) * 4), 0x00020000);
-
   // Cursor over the (q head of the group, query tile) pairs, advanced incrementally so
   // that a step costs a handful of scalar instructions: the tile's first row, the head's
   // Q / dO base pointers and the offset of its statistics.
   struct Cursor {
     int qt, i0;
     const T *q_head, *do_head;
-    int64_t stat_row;  // index of row 0 of this head in the statistics arrays
+    int stat_row;  // index of row 0 of this head in the statistics arrays
   };
   const int i_first = qt_lo * C::BM;
   // Every head's walk over the n_qt query tiles starts at tile qt_start and wraps around,
@@ -211,7 +208,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   const int h_first = hk * a.group + part * hpu;
   nxt.q_head = q_base + (int64_t)h_first * a.q_st[2];
   nxt.do_head = do_base + (int64_t)h_first * a.do_st[2];
-  nxt.stat_row = (int64_t)h_first * a.rows_q + ws_row0;
+  nxt.stat_row = (int)(h_first * a.rows_q + ws_row0);
   // The next tile is fetched by NPART instructions per wave (statistics, Q, dO), issued
   // one at a time between the first MFMAs of a step; advance() then moves the cursor on.
   constexpr int NQD = TileDma<D, C::BM, C::THREADS>::N;
@@ -219,23 +216,23 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   auto load_part = [&](int part, char* qd, char* dod, float* std_) __attribute__((always_inline)) {
     if (part == 0) {
       if (wave == 0) {  // lanes 0-31: lse2 of the 32 rows, lanes 32-63: their delta
-        const int soff = (int)((nxt.stat_row + nxt.i0) * 4);
+        const int first = nxt.stat_row + nxt.i0;
+        const __amdgpu_buffer_rsrc_t st_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            (void*)(a.lse2 + first), 0, min(stat_end - first, stat_elems + C::BM) * 4, 0x00020000);
         // the per-lane offset is recomputed here (opaque to the optimiser): kept in a
         // register across the walk it could be spilled, and its reload would wait for
         // every tile load issued before it
         int l = lane;
         asm volatile("" : "+v"(l));
-        const int voff = ((l & 31) << 2) + (l >> 5) * (int)(stat_elems * 4);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(st_rsrc, (lds_void_t*)std_, 4, voff, soff, 0, 0);
+        const int voff = ((l & 31) << 2) + (l >> 5) * (stat_elems * 4);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(st_rsrc, (lds_void_t*)std_, 4, voff, 0, 0, 0);
       }
     } else if (part <= NQD) {
-      const __amdgpu_buffer_rsrc_t q_rsrc =
-          __builtin_amdgcn_make_buffer_rsrc((void*)nxt.q_head, 0, q_extent, 0x00020000);
-      q_dma.load_one(q_rsrc, nxt.i0 * q_row_bytes, qd, part - 1);
+      const TileSrc t = tile_src<C::BM, FAR>(nxt.q_head, nxt.i0, len_q, q_row_bytes, C::ROWB);
+      q_dma.load_one(t.rsrc, t.soff, qd, part - 1);
     } else {
-      const __amdgpu_buffer_rsrc_t do_rsrc =
-          __builtin_amdgcn_make_buffer_rsrc((void*)nxt.do_head, 0, do_extent, 0x00020000);
-      do_dma.load_one(do_rsrc, nxt.i0 * do_row_bytes, dod, part - 1 - NQD);
+      const TileSrc t = tile_src<C::BM, FAR>(nxt.do_head, nxt.i0, len_q, do_row_bytes, C::ROWB);
+      do_dma.load_one(t.rsrc, t.soff, dod, part - 1 - NQD);
     }
   };
   auto advance = [&]() __attribute__((always_inline)) {
@@ -251,13 +248,13 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
       nxt.i0 = i_first + qt_start * C::BM;
       nxt.q_head += a.q_st[2];
       nxt.do_head += a.do_st[2];
-      nxt.stat_row += a.rows_q;
+      nxt.stat_row += (int)a.rows_q;
     }
   };
 
   if (n_iter > 0) {
-    const __amdgpu_buffer_rsrc_t v_rsrc = make_rows_rsrc(v_ptr, len_k, a.v_st[1] * 2, C::ROWB);
-    v_dma.load(v_rsrc, (int)(j0 * a.v_st[1] * 2), v_s);
+    // (once per block: always based at the tile)
+    v_dma.load(tile_src<C::BN, true>(v_ptr, j0, len_k, (int)(a.v_st[1] * 2), C::ROWB), v_s);
 #pragma unroll
     for (int part = 0; part < NPART; part++) load_part(part, q_s0, do_s0, st_s0);
     advance();
@@ -550,7 +547,7 @@ struct DqCfg {
 // of neighbouring key blocks, packed, are the B operand of dQ^T += K^T dS^T over a 32-key slab
 // (k order: four keys of the first block, then four of the second); the A operand follows the
 // same order: two transposing reads, one per key block.
-template <typename T, int D>
+template <typename T, int D, bool FAR>
 __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(const AttnArgs a) {
   using C = DqCfg<D>;
   using M = Mma<T>;
@@ -672,15 +669,14 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(const AttnArgs a) {
   const int rl = 4 * u + (r >> 2);
   const int t_row = rl * C::ROWB + ((((r & 3) >> 1) ^ swz16_f<C::CPR>(rl)) << 4) + (r & 1) * 8;
 
-  const __amdgpu_buffer_rsrc_t k_rsrc = make_rows_rsrc(k_ptr, len_k, a.k_st[1] * 2, C::ROWB);
-  const __amdgpu_buffer_rsrc_t v_rsrc = make_rows_rsrc(v_ptr, len_k, a.v_st[1] * 2, C::ROWB);
   TileDma<D, C::BN, C::THREADS, true> k_dma, v_dma;
   k_dma.init(a.k_st[1], tid);
   v_dma.init(a.v_st[1], tid);
-  const int k_tile_bytes = (int)(C::BN * a.k_st[1] * 2), v_tile_bytes = (int)(C::BN * a.v_st[1] * 2);
+  const int k_row_bytes = (int)(a.k_st[1] * 2), v_row_bytes = (int)(a.v_st[1] * 2);
   auto load_tile = [&](int it, char* kd, char* vd) __attribute__((always_inline)) {
-    k_dma.load(k_rsrc, tile_of(it) * k_tile_bytes, kd);
-    v_dma.load(v_rsrc, tile_of(it) * v_tile_bytes, vd);
+    const int j = tile_of(it) * C::BN;
+    k_dma.load(tile_src<C::BN, FAR>(k_ptr, j, len_k, k_row_bytes, C::ROWB), kd);
+    v_dma.load(tile_src<C::BN, FAR>(v_ptr, j, len_k, v_row_bytes, C::ROWB), vd);
   };
 
   auto step = [&](int it, const char* kc, const char* vc, char* kn,
@@ -896,9 +892,12 @@ __global__ __launch_bounds__(256) void attn_bwd_prep_kernel(const AttnArgs a) {
 // Explicit instantiations: with implicit instantiation alone this hipcc emits the host
 // launch stubs of only some of the variants.
 #define RSWA_INSTANTIATE(T, D)                                              \
-  template __global__ void attn_bwd_dkdv_kernel<T, D, false>(const AttnArgs); \
-  template __global__ void attn_bwd_dkdv_kernel<T, D, true>(const AttnArgs);  \
-  template __global__ void attn_bwd_dq_kernel<T, D>(const AttnArgs);        \
+  template __global__ void attn_bwd_dkdv_kernel<T, D, false, false>(const AttnArgs); \
+  template __global__ void attn_bwd_dkdv_kernel<T, D, true, false>(const AttnArgs);  \
+  template __global__ void attn_bwd_dkdv_kernel<T, D, false, true>(const AttnArgs);  \
+  template __global__ void attn_bwd_dkdv_kernel<T, D, true, true>(const AttnArgs);   \
+  template __global__ void attn_bwd_dq_kernel<T, D, false>(const AttnArgs);          \
+  template __global__ void attn_bwd_dq_kernel<T, D, true>(const AttnArgs);           \
   template __global__ void attn_bwd_prep_kernel<T, D>(const AttnArgs);
 RSWA_INSTANTIATE(__bf16, 128)
 RSWA_INSTANTIATE(__bf16, 64)
@@ -928,12 +927,13 @@ int launch_bwd(AttnArgs& a, hipStream_t stream, int phases) {
     }
     if (a.n_work > 0) {
       clear_launch_error();
+      const dim3 grid(padded_grid(a.n_work)), block(C::THREADS);
       if (a.nsplit > 1) {
-        hipLaunchKernelGGL((attn_bwd_dkdv_kernel<T, D, true>), dim3(padded_grid(a.n_work)),
-                           dim3(C::THREADS), 0, stream, a);
+        if (a.far) hipLaunchKernelGGL((attn_bwd_dkdv_kernel<T, D, true, true>), grid, block, 0, stream, a);
+        else hipLaunchKernelGGL((attn_bwd_dkdv_kernel<T, D, true, false>), grid, block, 0, stream, a);
       } else {
-        hipLaunchKernelGGL((attn_bwd_dkdv_kernel<T, D, false>), dim3(padded_grid(a.n_work)),
-                           dim3(C::THREADS), 0, stream, a);
+        if (a.far) hipLaunchKernelGGL((attn_bwd_dkdv_kernel<T, D, false, true>), grid, block, 0, stream, a);
+        else hipLaunchKernelGGL((attn_bwd_dkdv_kernel<T, D, false, false>), grid, block, 0, stream, a);
       }
       int rc = check_launch("attn_bwd dkdv");
       if (rc != RSWA_OK) return rc;
@@ -953,8 +953,9 @@ int launch_bwd(AttnArgs& a, hipStream_t stream, int phases) {
     }
     if (a.n_work > 0) {
       clear_launch_error();
-      hipLaunchKernelGGL((attn_bwd_dq_kernel<T, D>), dim3(padded_grid(a.n_work)),
-                         dim3(C::THREADS), 0, stream, a);
+      const dim3 grid(padded_grid(a.n_work)), block(C::THREADS);
+      if (a.far) hipLaunchKernelGGL((attn_bwd_dq_kernel<T, D, true>), grid, block, 0, stream, a);
+      else hipLaunchKernelGGL((attn_bwd_dq_kernel<T, D, false>), grid, block, 0, stream, a);
       int rc = check_launch("attn_bwd dq");
       if (rc != RSWA_OK) return rc;
     }

@@ -56,6 +56,7 @@ struct AttnArgs {
   // tiles (forward, dQ) or key tiles (dK/dV) so that the tiles with the most visible
   // pairs start first and the short ones fill the tail of the launch.
   int32_t rev_q, rev_k;
+  int32_t far;  // a sequence of some streamed tensor spans 2 GiB or more: FAR kernels
   float scale, scale_log2;
 };
 
@@ -259,6 +260,34 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rows_rsrc(const void* bas
   return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, (int)bytes, 0x00020000);
 }
 
+// Where the ROWS-row tile that starts at row `row0` of a slice of `rows` rows is fetched from:
+// a resource and the byte offset of the tile's first row inside it (rows past the slice's
+// last read as zero).
+//   FAR = false: the resource covers the whole slice (loop-invariant) and the offset selects the
+//                tile; the slice must span less than 2 GiB.
+//   FAR = true:  the resource is based at the tile's first row (64-bit pointer arithmetic, all
+//                else 32-bit scalar arithmetic) and covers the tile only, so that a slice may
+//                span any number of bytes as long as one tile spans less than 2 GiB.  Costs a
+//                dozen scalar instructions per tile (2 % of the dK/dV kernel, whose single wave
+//                per SIMD hides nothing), which is why the host picks it only when needed.
+struct TileSrc {
+  __amdgpu_buffer_rsrc_t rsrc;
+  int soff;
+};
+template <int ROWS, bool FAR>
+__device__ __forceinline__ TileSrc tile_src(const void* base, int row0, int rows, int stride_bytes,
+                                            int row_bytes) {
+  if constexpr (FAR) {
+    const int n = min(rows - row0, ROWS);  // rows of the tile that exist
+    const int bytes = n > 0 ? (n - 1) * stride_bytes + row_bytes : 0;
+    const uint64_t off = (uint64_t)(uint32_t)row0 * (uint64_t)(uint32_t)stride_bytes;
+    return {__builtin_amdgcn_make_buffer_rsrc((void*)((const char*)base + off), 0, bytes, 0x00020000),
+            0};
+  } else {
+    return {make_rows_rsrc(base, rows, stride_bytes, row_bytes), row0 * stride_bytes};
+  }
+}
+
 // Cooperative copy of a [ROWS x D] tile into a swizzled LDS tile with buffer loads that
 // land directly in LDS (buffer_load_dwordx4 ... lds: lane L of a wave writes
 // wave_base + 16 L).  The per-lane byte offsets are computed once (init); a tile load is
@@ -294,6 +323,9 @@ struct TileDma {
   __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t rsrc, int soff, char* lds_tile) const {
 #pragma unroll
     for (int n = 0; n < N; n++) load_one(rsrc, soff, lds_tile, n);
+  }
+  __device__ __forceinline__ void load(const TileSrc& t, char* lds_tile) const {
+    load(t.rsrc, t.soff, lds_tile);
   }
 };
 
@@ -339,6 +371,7 @@ __device__ __forceinline__ float halfwave_sum(float x) {
 // prologue, partial store and share of the final sum -- so launches that already give every
 // compute unit a block are left alone.
 constexpr int kDkvKeysPerBlock = 256;
+constexpr int kMaxTileRows = 256;  // most rows any kernel fetches as one tile (V in dK/dV)
 constexpr int kComputeUnits = 256;  // MI355X
 #ifndef RSWA_DKDV_SPLIT_BELOW
 #define RSWA_DKDV_SPLIT_BELOW (kComputeUnits / 2 + 1)

@@ -36,7 +36,7 @@ struct FwdCfg {
   static_assert(TILE >= 32 * O_STRIDE, "one wave's epilogue staging fits one tile buffer");
 };
 
-template <typename T, int D, bool SKIP>
+template <typename T, int D, bool SKIP, bool FAR>
 __global__ __launch_bounds__(512) void attn_fwd_kernel(const AttnArgs a) {
   using C = FwdCfg<D>;
   using M = Mma<T>;
@@ -141,17 +141,15 @@ __global__ __launch_bounds__(512) void attn_fwd_kernel(const AttnArgs a) {
   const int t_row1 = (rl + 8) * C::ROWB + ((lp ^ swz_f<C::CPR>(rl + 8)) << 4) + (i16 & 1) * 8;
 
   // ---- tile DMA: rows past len_k read as zero ---------------------------------
-  const __amdgpu_buffer_rsrc_t k_rsrc = make_rows_rsrc(k_ptr, len_k, a.k_st[1] * 2, C::ROWB);
-  const __amdgpu_buffer_rsrc_t v_rsrc = make_rows_rsrc(v_ptr, len_k, a.v_st[1] * 2, C::ROWB);
   TileDma<D, C::BN, C::THREADS> k_dma, v_dma;
   k_dma.init(a.k_st[1], tid);
   v_dma.init(a.v_st[1], tid);
-  const int k_tile_bytes = (int)(C::BN * a.k_st[1] * 2), v_tile_bytes = (int)(C::BN * a.v_st[1] * 2);
+  const int k_row_bytes = (int)(a.k_st[1] * 2), v_row_bytes = (int)(a.v_st[1] * 2);
   auto load_k = [&](int it, char* dst) __attribute__((always_inline)) {
-    k_dma.load(k_rsrc, tile_of(it) * k_tile_bytes, dst);
+    k_dma.load(tile_src<C::BN, FAR>(k_ptr, tile_of(it) * C::BN, len_k, k_row_bytes, C::ROWB), dst);
   };
   auto load_v = [&](int it, char* dst) __attribute__((always_inline)) {
-    v_dma.load(v_rsrc, tile_of(it) * v_tile_bytes, dst);
+    v_dma.load(tile_src<C::BN, FAR>(v_ptr, tile_of(it) * C::BN, len_k, v_row_bytes, C::ROWB), dst);
   };
 
   // ---- pieces of one tile ------------------------------------------------------
@@ -373,8 +371,10 @@ __global__ __launch_bounds__(512) void attn_fwd_kernel(const AttnArgs a) {
 // Explicit instantiations: with implicit instantiation alone this hipcc emits the host
 // launch stubs of only some of the four variants.
 #define RSWA_INSTANTIATE(T, D)                                               \
-  template __global__ void attn_fwd_kernel<T, D, false>(const AttnArgs);     \
-  template __global__ void attn_fwd_kernel<T, D, true>(const AttnArgs);
+  template __global__ void attn_fwd_kernel<T, D, false, false>(const AttnArgs); \
+  template __global__ void attn_fwd_kernel<T, D, true, false>(const AttnArgs);  \
+  template __global__ void attn_fwd_kernel<T, D, false, true>(const AttnArgs);  \
+  template __global__ void attn_fwd_kernel<T, D, true, true>(const AttnArgs);
 RSWA_INSTANTIATE(__bf16, 128)
 RSWA_INSTANTIATE(__bf16, 64)
 RSWA_INSTANTIATE(_Float16, 128)
@@ -400,12 +400,13 @@ int launch_fwd(AttnArgs& a, hipStream_t stream) {
   const int64_t span = (a.wl < 0 || a.wr < 0) ? (int64_t)1 << 40 : (int64_t)a.wl + a.wr + 1;
   const bool skip = (bm - 32) * 10 >= span + bm;
   clear_launch_error();
+  const dim3 grid(padded_grid(a.n_work)), block(C::THREADS);
   if (skip) {
-    hipLaunchKernelGGL((attn_fwd_kernel<T, D, true>), dim3(padded_grid(a.n_work)),
-                       dim3(C::THREADS), 0, stream, a);
+    if (a.far) hipLaunchKernelGGL((attn_fwd_kernel<T, D, true, true>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((attn_fwd_kernel<T, D, true, false>), grid, block, 0, stream, a);
   } else {
-    hipLaunchKernelGGL((attn_fwd_kernel<T, D, false>), dim3(padded_grid(a.n_work)),
-                       dim3(C::THREADS), 0, stream, a);
+    if (a.far) hipLaunchKernelGGL((attn_fwd_kernel<T, D, false, true>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((attn_fwd_kernel<T, D, false, false>), grid, block, 0, stream, a);
   }
   return check_launch("attn_fwd");
 }

@@ -71,7 +71,7 @@ class AttnParams(Structure):
         ("workspace", c_void_p),
         ("workspace_bytes", c_uint64),
         ("dq_accumulate", c_int32),
-        ("reserved_", c_int32),
+        ("addressing", c_int32),
     ]
 
 

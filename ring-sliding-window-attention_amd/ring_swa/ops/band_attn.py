@@ -19,6 +19,8 @@ visible key produce ``out = 0``, ``lse = -inf`` (the merge identity).
 """
 from __future__ import annotations
 
+import os
+
 from typing import Optional, Tuple
 
 import torch
@@ -91,6 +93,9 @@ def _params(q, k, v, softmax_scale, window_size, causal, cu_q, cu_k, num_sink,
     p.q_stride = _lib.i64x3(_strides3(q, packed))
     p.k_stride = _lib.i64x3(_strides3(k, packed))
     p.v_stride = _lib.i64x3(_strides3(v, packed))
+    # RSWA_ADDRESSING=far: the kernels that base every tile fetch at the tile's own first row
+    # (picked by the library itself once a sequence spans 2 GiB) whatever the sizes
+    p.addressing = 1 if os.environ.get("RSWA_ADDRESSING", "") == "far" else 0
     return p
 
 

@@ -97,3 +97,52 @@ def test_static_backward_refuses_oversize_without_a_gpu():
     rc = L.rswa_attn_bwd_static(p, None)
     assert rc == -2 and b"built-in" in L.rswa_last_error()
     assert L.rswa_attn_bwd_static(None, None) == -1
+
+
+def _fake_params(tokens, heads_q=32, heads_kv=8, d=128):
+    """Dense one-batch problem on placeholder addresses: enough for the argument checks,
+    which run before anything touches a device."""
+    from ring_swa import _lib
+
+    p = _lib.AttnParams()
+    p.dtype, p.head_dim, p.batch, p.heads_q, p.heads_kv = 0, d, 1, heads_q, heads_kv
+    p.seqlen_q = p.seqlen_k = tokens
+    p.softmax_scale = d ** -0.5
+    p.window_left, p.window_right, p.causal = 1024, 0, 1
+    for name in ("q", "k", "v", "out", "lse", "dout", "dq", "dk", "dv", "workspace"):
+        setattr(p, name, 4096)
+    rq, rk = (heads_q * d, d), (heads_kv * d, d)
+    for name, (row, head) in (("q", rq), ("k", rk), ("v", rk), ("out", rq), ("dout", rq),
+                              ("dq", rq), ("dk", rk), ("dv", rk)):
+        setattr(p, name + "_stride", _lib.i64x3((tokens * row, row, head)))
+    p.lse_stride = _lib.i64x3((heads_q * tokens, tokens, 1))
+    return p
+
+
+def test_what_stays_refused_beyond_2_gib_says_why():
+    """A sequence may span any number of bytes; what the 32-bit tile offsets still cannot
+    serve is refused with a message that names the limit."""
+    _ensure_built()
+    from ring_swa import _lib
+
+    L = _lib.lib()
+    # rows 4 MiB apart: one 256-row tile would span 2 GiB
+    p = _fake_params(1024)
+    p.k_stride = _lib.i64x3((0, 1 << 22, 128))
+    assert L.rswa_attn_fwd(p, None) == -2
+    assert b"row stride" in L.rswa_last_error()
+    p = _fake_params(1024)
+    p.dout_stride = _lib.i64x3((0, 1 << 22, 128))
+    p.workspace_bytes = L.rswa_attn_bwd_workspace_bytes(p)
+    assert L.rswa_attn_bwd(p, None) == -2
+    assert b"row stride of dout" in L.rswa_last_error()
+    # 2^24 + ... rows x 32 heads: each statistics array of the backward would reach 2 GiB
+    p = _fake_params(1 << 24)
+    p.workspace_bytes = L.rswa_attn_bwd_workspace_bytes(p)
+    assert L.rswa_attn_bwd(p, None) == -2
+    assert b"statistics array" in L.rswa_last_error()
+    # a little below that limit passes the size checks: the workspace is next
+    p = _fake_params((1 << 24) - 1024)
+    p.workspace_bytes = 0
+    assert L.rswa_attn_bwd(p, None) == -1
+    assert b"workspace" in L.rswa_last_error()
