@@ -102,7 +102,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   SeqInfo s;
   int kt;
   if (a.cu_q) {
-    if (!locate_packed(a, slot, C::BN, true, s, kt)) return;
+    static_assert(C::BN == 1 << 8, "tile size passed to locate_packed");
+    if (!locate_packed(a, slot, 8, true, s, kt)) return;
   } else {
     s.batch_idx = rest / a.heads_kv;
     s.q_row0 = s.k_row0 = 0;
@@ -580,7 +581,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(const AttnArgs a) {
   SeqInfo s;
   int qt;
   if (a.cu_q) {
-    if (!locate_packed(a, slot, bm, false, s, qt)) return;
+    if (!locate_packed(a, slot, pair ? 7 : 8, false, s, qt)) return;
   } else {
     s.batch_idx = rest / a.heads_kv;
     s.q_row0 = s.k_row0 = 0;

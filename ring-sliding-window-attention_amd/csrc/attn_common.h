@@ -93,29 +93,34 @@ __device__ __forceinline__ RowBounds row_bounds(const AttnArgs& a, int i, int le
   return r;
 }
 
-// Locate tile `t` (counted along the sequence axis `which`: 0 = q, 1 = k) of
-// granularity `tile` in packed mode.  Returns false if t is past the last tile.
-__device__ __forceinline__ bool locate_packed(const AttnArgs& a, int t, int tile, bool along_k,
+// Packed mode: which sequence, and which of its tiles of `tile` = 2^tile_log2 rows, does
+// tile slot `t` along the q or k axis stand for?  Sequence b owns the slots from
+// cu[b] / tile + b on -- strictly increasing in b, so a binary search over cu finds b in
+// log2(batch) dependent loads, where a running count of tiles would have to walk every
+// sequence before it.  ceil(len_b / tile) of its slots are its tiles; at most one more, before
+// the next sequence's first, stays unused (false is returned for it), which is why a packed
+// grid has ceil(rows / tile) + batch slots.
+__device__ __forceinline__ bool locate_packed(const AttnArgs& a, int t, int tile_log2, bool along_k,
                                               SeqInfo& s, int& tile_in_seq) {
   const int32_t* cu = along_k ? a.cu_k : a.cu_q;
-  int acc = 0;
-  for (int b = 0; b < a.batch; b++) {
-    const int len = cu[b + 1] - cu[b];
-    const int nt = (len + tile - 1) / tile;
-    if (t < acc + nt) {
-      s.batch_idx = b;
-      s.q_row0 = a.cu_q[b];
-      s.k_row0 = a.cu_k[b];
-      s.len_q = a.cu_q[b + 1] - a.cu_q[b];
-      s.len_k = a.cu_k[b + 1] - a.cu_k[b];
-      s.q_base = 0;
-      s.k_base = 0;
-      tile_in_seq = t - acc;
-      return true;
-    }
-    acc += nt;
+  int lo = 0, hi = a.batch;  // first slot of lo <= t; hi == batch or first slot of hi > t
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if ((cu[mid] >> tile_log2) + mid <= t) lo = mid;
+    else hi = mid;
   }
-  return false;
+  const int b = lo;
+  const int first = cu[b];
+  tile_in_seq = t - ((first >> tile_log2) + b);
+  if ((tile_in_seq << tile_log2) >= cu[b + 1] - first) return false;
+  s.batch_idx = b;
+  s.q_row0 = a.cu_q[b];
+  s.k_row0 = a.cu_k[b];
+  s.len_q = a.cu_q[b + 1] - a.cu_q[b];
+  s.len_k = a.cu_k[b + 1] - a.cu_k[b];
+  s.q_base = 0;
+  s.k_base = 0;
+  return true;
 }
 
 template <typename T>

@@ -71,7 +71,7 @@ __global__ __launch_bounds__(512) void attn_fwd_kernel(const AttnArgs a) {
   SeqInfo s;
   int qt;
   if (a.cu_q) {
-    if (!locate_packed(a, slot, bm, false, s, qt)) return;
+    if (!locate_packed(a, slot, pair ? 7 : 8, false, s, qt)) return;
   } else {
     s.batch_idx = rest / a.heads_kv;
     s.q_row0 = s.k_row0 = 0;

@@ -169,16 +169,20 @@ def test_config4_varlen_rank_slices_total32768_window2048():
         assert torch.isfinite(t.float()).all()
 
 
-@pytest.mark.parametrize("impl,n_sink", [("split", 4), ("fused", 4), ("split", 1)])
-def test_config5_streaming_llm_varlen_total65536_sinks(impl, n_sink):
+@pytest.mark.parametrize("impl,n_sink,off", [("split", 4, 0), ("fused", 4, 0), ("split", 1, 0),
+                                             ("fused", 4, 37), ("split", 4, 37), ("fused", 1, 37)])
+def test_config5_streaming_llm_varlen_total65536_sinks(impl, n_sink, off):
     """n_sink = 4: the configuration as stated (keyword-only extension of the API);
-    n_sink = 1: the reference's own single sink through the unchanged signature."""
+    n_sink = 1: the reference's own single sink through the unchanged signature.
+    off = 0: sequence boundaries on multiples of 1024, hence on the kernels' tile edges;
+    off = 37: boundaries at 1024 c + 37, + 101, + 165 -- inside 32-, 64-, 128- and 256-row tiles."""
     import ring_swa
 
     total, hq, hk, w = 65536, 32, 8, 4092
     g = torch.Generator().manual_seed(0)
     cuts = sorted((torch.randperm(total // 1024 - 1, generator=g)[:3] + 1).tolist())
-    cu = [0] + [c * 1024 for c in cuts] + [total]
+    cu = [0] + [c * 1024 + (off + 64 * i if off else 0) for i, c in enumerate(cuts)] + [total]
+    assert all((c % 32 != 0) for c in cu[1:-1]) or off == 0
     q, do = _randn((total, hq, D), 0), _randn((total, hq, D), 1)
     k, v = _randn((total, hk, D), 2), _randn((total, hk, D), 3)
     for c in cu[:-1]:
