@@ -145,6 +145,11 @@ struct Mma<__bf16> {
   // its result, copies added by the register allocator included -- accumulators that live
   // across control flow are therefore better served by the builtin.  Volatile: they keep
   // their order among themselves and the empty volatile statements that pin vector work.
+  // RSWA_MFMA_BUILTIN_ONLY builds the same three through the builtin instead: the compiler then
+  // pads every hazard itself (and is free to place the accumulators badly).  The build makes a
+  // second library that way, and a GPU test holds the two to the same output bits -- a
+  // scheduler change in a later compiler that broke the distance kept by hand would show there.
+#ifndef RSWA_MFMA_BUILTIN_ONLY
   static __device__ __forceinline__ void mfma32_vec(V8 a, V8 b, f32x16& c) {
     asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
   }
@@ -155,6 +160,15 @@ struct Mma<__bf16> {
   static __device__ __forceinline__ void mfma32_vec_init(V8 a, V8 b, const f32x16& init, f32x16& c) {
     asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3" : "=&v"(c) : "v"(a), "v"(b), "v"(init));
   }
+#else
+  static __device__ __forceinline__ void mfma32_vec(V8 a, V8 b, f32x16& c) { c = mfma32(a, b, c); }
+  static __device__ __forceinline__ void mfma32_vec0(V8 a, V8 b, f32x16& c) {
+    c = mfma32(a, b, f32x16{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0});
+  }
+  static __device__ __forceinline__ void mfma32_vec_init(V8 a, V8 b, const f32x16& init, f32x16& c) {
+    c = mfma32(a, b, init);
+  }
+#endif
   static __device__ __forceinline__ V8 pack(const float* x) {
     f32x8 f = {x[0], x[1], x[2], x[3], x[4], x[5], x[6], x[7]};
     return __builtin_convertvector(f, V8);
@@ -175,6 +189,7 @@ struct Mma<_Float16> {
   static __device__ __forceinline__ f32x4 mfma16(V8 a, V8 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
   }
+#ifndef RSWA_MFMA_BUILTIN_ONLY
   static __device__ __forceinline__ void mfma32_vec(V8 a, V8 b, f32x16& c) {
     asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
   }
@@ -185,6 +200,15 @@ struct Mma<_Float16> {
   static __device__ __forceinline__ void mfma32_vec_init(V8 a, V8 b, const f32x16& init, f32x16& c) {
     asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %3" : "=&v"(c) : "v"(a), "v"(b), "v"(init));
   }
+#else
+  static __device__ __forceinline__ void mfma32_vec(V8 a, V8 b, f32x16& c) { c = mfma32(a, b, c); }
+  static __device__ __forceinline__ void mfma32_vec0(V8 a, V8 b, f32x16& c) {
+    c = mfma32(a, b, f32x16{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0});
+  }
+  static __device__ __forceinline__ void mfma32_vec_init(V8 a, V8 b, const f32x16& init, f32x16& c) {
+    c = mfma32(a, b, init);
+  }
+#endif
   static __device__ __forceinline__ V8 pack(const float* x) {
     f32x8 f = {x[0], x[1], x[2], x[3], x[4], x[5], x[6], x[7]};
     return __builtin_convertvector(f, V8);

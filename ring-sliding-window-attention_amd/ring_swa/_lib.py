@@ -92,7 +92,13 @@ def lib() -> ctypes.CDLL:
             f"`python {os.path.join(_PKG_ROOT, 'build.py')}` (needs hipcc; no GPU required). "
             "ring_swa has no non-HIP fallback."
         )
-    L = ctypes.CDLL(LIB_PATH)
+    _lib = load(LIB_PATH)
+    return _lib
+
+
+def load(path: str) -> ctypes.CDLL:
+    """Open a build of the library and declare its entry points."""
+    L = ctypes.CDLL(path)
     L.rswa_last_error.restype = c_char_p
     L.rswa_last_error.argtypes = []
     L.rswa_version.restype = c_int
@@ -119,7 +125,6 @@ def lib() -> ctypes.CDLL:
             f"({L.rswa_sizeof_attn_params()} bytes) and the Python binding "
             f"({ctypes.sizeof(AttnParams)} bytes): rebuild the library"
         )
-    _lib = L
     return L
 
 
