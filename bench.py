@@ -143,6 +143,107 @@ def global_pairs_of_rows(cu, w, row0, row1, n_sink=0):
     return total
 
 
+def _mk(dev):
+    import torch
+
+    return lambda *shape: torch.randn(*shape, device=dev, dtype=torch.bfloat16)
+
+
+def case_c2(dev):
+    """Configuration 2: plain single-GPU sliding-window attention, batch 2, seq 8192, 32 q = 32
+    kv heads, head_dim 128, window 1000.  Returns (forward, backward, pairs x batch x heads)."""
+    import torch
+
+    from ring_swa.ops import attn_bwd, attn_fwd
+
+    mk = _mk(dev)
+    q2, k2, v2, do2 = (mk(2, 8192, 32, 128) for _ in range(4))
+    o2, l2 = attn_fwd(q2, k2, v2, None, (1000, 0), True)
+    g2 = [torch.empty_like(q2) for _ in range(3)]
+    fwd = lambda: attn_fwd(q2, k2, v2, None, (1000, 0), True)  # noqa: E731
+    bwd = lambda: attn_bwd(q2, k2, v2, o2, l2, do2, *g2, None, (1000, 0), True)  # noqa: E731
+    return fwd, bwd, band_pairs(8192, 1000) * 2 * 32
+
+
+def case_c4(dev):
+    """Configuration 4: a pack of 32768 tokens (log-uniform lengths in [64, 16384], seed 0),
+    32 q / 8 kv heads, head_dim 128, window 2048.  Two steps (forward + backward): one rank
+    slice of virtual cp 4 whose chunk starts inside a sequence (diagonal packed block +
+    rectangle on the previous chunk + merge), and the whole pack in one call."""
+    import itertools
+
+    import torch
+
+    import ring_swa
+
+    mk = _mk(dev)
+    T4, CP4, W4, HQ, HK, D = 32768, 4, 2048, 32, 8, 128
+    lens4 = log_uniform_lengths(T4, 64, 16384, seed=0)
+    cu4 = [0] + list(itertools.accumulate(lens4))
+    s4 = T4 // CP4
+    r4 = next(r for r in range(1, CP4) if (r * s4) not in cu4)
+    q4, do4 = mk(T4, HQ, D), mk(T4, HQ, D)
+    k4, v4 = mk(T4, HK, D), mk(T4, HK, D)
+    sl = slice(r4 * s4, (r4 + 1) * s4)
+    ps = slice((r4 - 1) * s4, r4 * s4)
+    qr, kr, vr = (t[sl].clone().requires_grad_() for t in (q4, k4, v4))
+    pr = torch.stack([k4[ps], v4[ps]]).requires_grad_()
+    do_r = do4[sl]
+
+    @torch.enable_grad()
+    def c4_slice():
+        for t in (qr, kr, vr, pr):
+            t.grad = None
+        ring_swa.ring_rank_share_attn_varlen(qr, kr, vr, [pr], W4, cu4, CP4, r4).backward(do_r)
+
+    cu4_dev = torch.tensor(cu4, dtype=torch.int32, device=dev)
+    qg4, kg4, vg4 = (t.clone().requires_grad_() for t in (q4, k4, v4))
+
+    @torch.enable_grad()
+    def c4_whole():
+        for t in (qg4, kg4, vg4):
+            t.grad = None
+        ring_swa.ring_sliding_window_attn_varlen(qg4, kg4, vg4, W4, cu4_dev, cp_size=1).backward(do4)
+
+    info = {"sequences": len(lens4), "rank": r4,
+            "pairs_slice": global_pairs_of_rows(cu4, W4, r4 * s4, (r4 + 1) * s4),
+            "pairs_whole": sum(band_pairs(n, W4) for n in lens4)}
+    return c4_slice, c4_whole, info
+
+
+def case_c5(dev, impl, n_sink):
+    """Configuration 5: packed streaming-LLM attention, 65536 tokens in 4 sequences (cut points
+    inside the kernels' tiles), 32 q / 8 kv heads, head_dim 128, sinks + window 4092, sink keys
+    scaled by 4.  Returns the forward + backward step and its pair count."""
+    import torch
+
+    import ring_swa
+
+    mk = _mk(dev)
+    T5, W5, HQ, HK, D = 65536, 4092, 32, 8, 128
+    g5 = torch.Generator().manual_seed(0)
+    cuts = sorted((torch.randperm(T5 // 1024 - 1, generator=g5)[:3] + 1).tolist())
+    cu5 = [0] + [c * 1024 + 37 + 64 * i for i, c in enumerate(cuts)] + [T5]
+    lens5 = [b - a for a, b in zip(cu5[:-1], cu5[1:])]
+    cu5_dev = torch.tensor(cu5, dtype=torch.int32, device=dev)
+    torch.manual_seed(5)
+    q5, do5 = mk(T5, HQ, D), mk(T5, HQ, D)
+    k5, v5 = mk(T5, HK, D), mk(T5, HK, D)
+    for c in cu5[:-1]:
+        k5[c:c + n_sink] *= 4
+    qg, kg, vg = (t.requires_grad_() for t in (q5, k5, v5))
+    kw = {} if n_sink == 1 else {"num_sink_tokens": n_sink}
+
+    @torch.enable_grad()
+    def c5_step():
+        for t in (qg, kg, vg):
+            t.grad = None
+        ring_swa.ring_streaming_llm_attn_varlen(qg, kg, vg, W5, cu5_dev, cp_size=1, impl=impl,
+                                                **kw).backward(do5)
+
+    return c5_step, {"lengths": lens5, "pairs": global_pairs_of_rows(cu5, W5, 0, T5, n_sink)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -153,6 +254,9 @@ def main():
     ap.add_argument("--pmc-pass", action="store_true",
                     help="counter-collection pass: launch a 1 GiB device copy (the known-size "
                          "calibration kernel) and every hot kernel twice, then exit")
+    ap.add_argument("--trace", choices=["c2", "c4", "c5"],
+                    help="kernel-trace pass: run only that configuration's step a few times "
+                         "(under rocprofv3 --kernel-trace --stats) and exit")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build covers the single-GPU path only; run with --gpus 1 "
@@ -190,6 +294,21 @@ def main():
             t.grad = None
         out = ring_swa.ring_rank_share_attn(q, k, v, [prev], W, CP, RANK)
         out.backward(do)
+
+    if args.trace:
+        if args.trace == "c2":
+            f2, b2, _ = case_c2(dev)
+            steps = [lambda: (f2(), b2())]
+        elif args.trace == "c4":
+            steps = list(case_c4(dev)[:2])
+        else:
+            steps = [case_c5(dev, "fused", 4)[0]]
+        for fn in steps:
+            for _ in range(args.steps):
+                fn()
+        torch.cuda.synchronize()
+        print(json.dumps({"trace_pass": args.trace, "steps": args.steps}))
+        return
 
     if args.pmc_pass:
         with torch.no_grad():
@@ -336,97 +455,34 @@ def main():
                 "ms": pair_med, "TFLOP/s": tf(8 * D * pairs * HQ, pair_med),
                 "pct_bf16_mfma_peak": 100.0 * tf(8 * D * pairs * HQ, pair_med) / PEAK_BF16_TFLOPS,
                 "flops_per_pair": "8 D", "note": "two launches on two streams, as in the rank step"}
-            # config 2: plain single-GPU SWA, batch 2, seq 8192, 32/32 heads, window 1000
-            q2, k2, v2, do2 = (mk(2, 8192, 32, 128) for _ in range(4))
-            o2, l2 = attn_fwd(q2, k2, v2, None, (1000, 0), True)
-            g2 = [torch.empty_like(q2) for _ in range(3)]
-            f2, _ = event_ms(lambda: attn_fwd(q2, k2, v2, None, (1000, 0), True), 10)
-            b2, _ = event_ms(lambda: attn_bwd(q2, k2, v2, o2, l2, do2, *g2, None, (1000, 0), True), 10)
-            p2 = band_pairs(8192, 1000) * 2 * 32
+            # the other GPU configurations of the suite (see the case_* functions)
+            f2, b2, p2 = case_c2(dev)
+            f2_ms, _ = event_ms(f2, 10)
+            b2_ms, _ = event_ms(b2, 10)
             rec["c2_swa_b2_s8192_h32_w1000"] = {
-                "fwd_ms": f2, "bwd_ms": b2, "TFLOP/s": 14 * 128 * p2 / (f2 + b2) / 1e9,
-                "pct_bf16_mfma_peak": 14 * 128 * p2 / (f2 + b2) / 1e9 / PEAK_BF16_TFLOPS * 100}
-            del q2, k2, v2, do2, o2, l2, g2
-            # config 4: packed pack of 32768 tokens (log-uniform lengths), window 2048; one rank
-            # slice of virtual cp 4 whose chunk starts inside a sequence (diagonal packed block +
-            # rectangle on the previous chunk + merge), and the whole pack in one call
-            import itertools
-
-            T4, CP4, W4 = 32768, 4, 2048
-            lens4 = log_uniform_lengths(T4, 64, 16384, seed=0)
-            cu4 = [0] + list(itertools.accumulate(lens4))
-            s4 = T4 // CP4
-            r4 = next(r for r in range(1, CP4) if (r * s4) not in cu4)
-            q4, do4 = mk(T4, HQ, D), mk(T4, HQ, D)
-            k4, v4 = mk(T4, HK, D), mk(T4, HK, D)
-            sl = slice(r4 * s4, (r4 + 1) * s4)
-            ps = slice((r4 - 1) * s4, r4 * s4)
-            qr, kr, vr = (t[sl].clone().requires_grad_() for t in (q4, k4, v4))
-            pr = torch.stack([k4[ps], v4[ps]]).requires_grad_()
-
-            @torch.enable_grad()
-            def c4_slice():
-                for t in (qr, kr, vr, pr):
-                    t.grad = None
-                ring_swa.ring_rank_share_attn_varlen(qr, kr, vr, [pr], W4, cu4, CP4, r4).backward(do4[sl])
-
-            cu4_dev = torch.tensor(cu4, dtype=torch.int32, device=dev)
-            qg4, kg4, vg4 = (t.clone().requires_grad_() for t in (q4, k4, v4))
-
-            @torch.enable_grad()
-            def c4_whole():
-                for t in (qg4, kg4, vg4):
-                    t.grad = None
-                ring_swa.ring_sliding_window_attn_varlen(qg4, kg4, vg4, W4, cu4_dev, cp_size=1).backward(do4)
-
+                "fwd_ms": f2_ms, "bwd_ms": b2_ms, "TFLOP/s": tf(14 * 128 * p2, f2_ms + b2_ms),
+                "pct_bf16_mfma_peak": tf(14 * 128 * p2, f2_ms + b2_ms) / PEAK_BF16_TFLOPS * 100}
+            del f2, b2
+            c4_slice, c4_whole, info4 = case_c4(dev)
             t_slice, _ = event_ms(c4_slice, 10)
             t_whole, _ = event_ms(c4_whole, 10)
-            p_slice = global_pairs_of_rows(cu4, W4, r4 * s4, (r4 + 1) * s4)
-            p_whole = sum(band_pairs(l, W4) for l in lens4)
+            rate = lambda p_, t_: {"ms": t_, "pairs_per_head": p_, "TFLOP/s": tf(14 * D * p_ * HQ, t_),  # noqa: E731
+                                   "pct_bf16_mfma_peak": tf(14 * D * p_ * HQ, t_) / PEAK_BF16_TFLOPS * 100}
             rec["c4_varlen_t32768_w2048"] = {
-                "sequences": len(lens4), "rank": r4,
-                "rank_slice": {"ms": t_slice, "pairs_per_head": p_slice,
-                               "TFLOP/s": tf(14 * D * p_slice * HQ, t_slice),
-                               "pct_bf16_mfma_peak": tf(14 * D * p_slice * HQ, t_slice) / PEAK_BF16_TFLOPS * 100},
-                "whole_pack_one_call": {"ms": t_whole, "pairs_per_head": p_whole,
-                                        "TFLOP/s": tf(14 * D * p_whole * HQ, t_whole),
-                                        "pct_bf16_mfma_peak": tf(14 * D * p_whole * HQ, t_whole) / PEAK_BF16_TFLOPS * 100}}
-            del q4, k4, v4, do4, qr, kr, vr, pr, qg4, kg4, vg4
-            # config 5: packed streaming-LLM, 65536 tokens in 4 sequences (cut points not
-            # multiples of the kernels' tiles), sinks + window 4092, sink keys x4
-            T5, W5 = 65536, 4092
-            g5 = torch.Generator().manual_seed(0)
-            cuts = sorted((torch.randperm(T5 // 1024 - 1, generator=g5)[:3] + 1).tolist())
-            cu5 = [0] + [c * 1024 + 37 + 64 * i for i, c in enumerate(cuts)] + [T5]
-            lens5 = [b - a for a, b in zip(cu5[:-1], cu5[1:])]
-            cu5_dev = torch.tensor(cu5, dtype=torch.int32, device=dev)
-            q5, do5 = mk(T5, HQ, D), mk(T5, HQ, D)
-            k5, v5 = mk(T5, HK, D), mk(T5, HK, D)
-            c5 = {"lengths": lens5}
+                "sequences": info4["sequences"], "rank": info4["rank"],
+                "rank_slice": rate(info4["pairs_slice"], t_slice),
+                "whole_pack_one_call": rate(info4["pairs_whole"], t_whole)}
+            del c4_slice, c4_whole
+            c5 = {}
             for n_sink in (1, 4):
-                kk5 = k5.clone()
-                for c in cu5[:-1]:
-                    kk5[c:c + n_sink] *= 4
-                pairs5 = global_pairs_of_rows(cu5, W5, 0, T5, n_sink) if n_sink == 4 else \
-                    sum(band_pairs(l, W5) + max(0, l - 1 - W5) for l in lens5)
                 for impl in ("fused", "split"):
-                    qg, kg, vg = (t.clone().requires_grad_() for t in (q5, kk5, v5))
-                    kw = {} if n_sink == 1 else {"num_sink_tokens": n_sink}
-
-                    @torch.enable_grad()
-                    def c5_step():
-                        for t in (qg, kg, vg):
-                            t.grad = None
-                        ring_swa.ring_streaming_llm_attn_varlen(qg, kg, vg, W5, cu5_dev, cp_size=1,
-                                                                impl=impl, **kw).backward(do5)
-
+                    c5_step, info5 = case_c5(dev, impl, n_sink)
                     t5, _ = event_ms(c5_step, 5, warm=2)
-                    c5[f"{impl}_sinks{n_sink}"] = {
-                        "ms": t5, "pairs_per_head": pairs5, "TFLOP/s": tf(14 * D * pairs5 * HQ, t5),
-                        "pct_bf16_mfma_peak": tf(14 * D * pairs5 * HQ, t5) / PEAK_BF16_TFLOPS * 100}
-                    del qg, kg, vg
+                    c5["lengths"] = info5["lengths"]
+                    c5[f"{impl}_sinks{n_sink}"] = rate(info5["pairs"], t5)
+                    del c5_step
             rec["c5_slm_varlen_t65536_w4092"] = c5
-            del q5, k5, v5, do5, kk5
+            T5 = 65536
             # the merge of that configuration's split path: all tokens x 32 heads, 16-bit
             # outputs and fp32 LSE on both sides (780 bytes per row)
             acc = torch.randn(1, T5, HQ, D, device=dev).bfloat16()
