@@ -31,15 +31,25 @@ BwdLayout bwd_layout(const rswa_attn_params* p, bool allow_split) {
         break;
       }
   }
-  L.count_off = 2 * L.stats_bytes;
-  L.part_off = L.count_off;
-  L.total_bytes = 2 * L.stats_bytes;
-  if (L.nsplit > 1) {
-    L.n_count = (int)blocks;
-    L.part_off = L.count_off + align_up((uint64_t)blocks * sizeof(int32_t), 256);
-    const uint64_t per_unit = (uint64_t)kDkvKeysPerBlock * p->head_dim * 2 * sizeof(float);
-    L.total_bytes = L.part_off + (uint64_t)blocks * L.nsplit * per_unit;
+  // Sink keys under a bounded window: the sink kernel, one chunk per ~512 rows of an average
+  // sequence (at most 64), one arrival counter per (sequence, kv head).
+  int64_t sink_units = 0;
+  if (p->num_sink > 0 && p->window_left >= 0) {
+    const int64_t rows_q = packed ? p->total_q / p->batch : p->seqlen_q;
+    L.sink_chunks = (int)std::min<int64_t>(64, std::max<int64_t>(1, (rows_q + 511) / 512));
+    sink_units = (int64_t)p->batch * p->heads_kv;
   }
+  // workspace: statistics | arrival counters (split key tiles, then sink units) | partial
+  // dK / dV of split key tiles | sums of the sink kernel
+  const int64_t split_units = L.nsplit > 1 ? blocks : 0;
+  L.n_count = (int)(split_units + sink_units);
+  L.sink_count_index = (int)split_units;
+  L.count_off = 2 * L.stats_bytes;
+  L.part_off = L.count_off + align_up((uint64_t)L.n_count * sizeof(int32_t), 256);
+  const uint64_t per_unit = (uint64_t)kDkvKeysPerBlock * p->head_dim * 2 * sizeof(float);
+  L.sink_off = L.part_off + (uint64_t)split_units * L.nsplit * per_unit;
+  L.total_bytes = L.sink_off + (uint64_t)sink_units * L.sink_chunks * p->num_sink * 2 * p->head_dim *
+                                   sizeof(float);
   return L;
 }
 
@@ -112,6 +122,9 @@ int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a, bool allow_
   a.dkv_count = nullptr;
   a.nsplit = 1;
   a.n_count = 0;
+  a.sink_part = nullptr;
+  a.sink_count = nullptr;
+  a.sink_chunks = 0;
   a.cu_q = p->cu_seqlens_q;
   a.cu_k = p->cu_seqlens_k;
   for (int i = 0; i < 3; i++) {
@@ -191,6 +204,9 @@ int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a, bool allow_
     a.n_count = L.n_count;
     a.dkv_count = (int32_t*)((char*)p->workspace + L.count_off);
     a.dkv_part = (float*)((char*)p->workspace + L.part_off);
+    a.sink_chunks = L.sink_chunks;
+    a.sink_part = L.sink_chunks ? (float*)((char*)p->workspace + L.sink_off) : nullptr;
+    a.sink_count = a.dkv_count + L.sink_count_index;
     // one load reaches from a row's lse2 to its delta, one array further on
     RSWA_REQUIRE(delta_bytes(p) < (1ull << 31) - 65536, RSWA_ERR_UNSUPPORTED,
                  "attn_bwd: rows * heads_q = %lld: each statistics array must stay below 2 GiB "

@@ -127,7 +127,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   // ---- query tiles that can see this key tile -------------------------------
   const int i_min = (a.wr >= 0) ? max(0, j0 - shift - a.wr) : 0;
   const int i_max =
-      (a.wl >= 0 && j0 >= a.n_sink) ? min(len_q - 1, j_last - shift + a.wl) : len_q - 1;
+      (a.wl >= 0) ? min(len_q - 1, j_last - shift + a.wl) : len_q - 1;
   const int qt_lo = i_min / C::BM;
   const int n_qt = (i_max >= i_min) ? i_max / C::BM - qt_lo + 1 : 0;
   const int n_iter = n_qt * hpu;
@@ -172,7 +172,6 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
         dk_acc[kb][d][i] = 0.f;
         dv_acc[kb][d][i] = 0.f;
       }
-
   // ---- tile DMA (rows past the end of the sequence read as zero) ------------------
   TileDma<D, C::BN, C::THREADS> v_dma;
   TileDma<D, C::BM, C::THREADS> q_dma, do_dma;
@@ -268,16 +267,15 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   // For which first rows i0 of a 32-row tile does any (query, key of this wave) pair survive
   // the mask (need_*), and for which is no pair masked (full_*)?  With
   // i1 = min(i0 + 32, len_q) - 1 and the wave's keys jw0 .. jw1 the conditions
-  //   needed: i0 < len_q, jw0 < len_k, jw0 <= i1 + shift + wr, (jw1 >= i0 + shift - wl or sink)
-  //   full:   i0 + 31 < len_q, jw1 < len_k, jw1 <= i0 + shift + wr,
-  //           (jw0 >= i0 + 31 + shift - wl or all the wave's keys are sinks)
+  //   needed: i0 < len_q, jw0 < len_k, jw0 <= i1 + shift + wr, jw1 >= i0 + shift - wl
+  //   full:   i0 + 31 < len_q, jw1 < len_k, jw1 <= i0 + shift + wr, jw0 >= i0 + 31 + shift - wl
   // are intervals of i0 whose ends depend on the wave only: a step tests two of them.
   constexpr int kInf = 1 << 30;
   int need_lo = (a.wr < 0) ? -kInf : jw0 - shift - a.wr - 31;
-  int need_hi = min(len_q - 1, (a.wl < 0 || jw0 < a.n_sink) ? kInf : jw1 - shift + a.wl);
+  int need_hi = min(len_q - 1, (a.wl < 0) ? kInf : jw1 - shift + a.wl);
   if (jw0 >= len_k || (a.wr >= 0 && len_q - 1 < jw0 - shift - a.wr)) need_hi = -kInf - 1;
   int full_lo = (a.wr < 0) ? -kInf : jw1 - shift - a.wr;
-  int full_hi = min(len_q - 32, (a.wl < 0 || jw1 < a.n_sink) ? kInf : jw0 - 31 - shift + a.wl);
+  int full_hi = min(len_q - 32, (a.wl < 0) ? kInf : jw0 - 31 - shift + a.wl);
   if (jw1 >= len_k) full_hi = -kInf - 1;
 
   // one query tile: prefetch the next one into (qn, don, stn), compute on (qc, doc, stc)
@@ -355,7 +353,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
           // key position relative to the aligned diagonal of row i0: rel(r) = rel0 - r
           const int jc = jw0 + kb * 32 + l32;
           const int rel0 = jc - i0 - shift;
-          const int rel_lo = (a.wl < 0 || jc < a.n_sink) ? -kInf : -a.wl;
+          const int rel_lo = (a.wl < 0) ? -kInf : -a.wl;
           const int rows_ok = (jc < len_k) ? len_q - i0 : 0;  // rows r < rows_ok are real
 #pragma unroll
           for (int e = 0; e < 4; e++) {
@@ -511,6 +509,188 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
       emit(grp / (KB * DB * 4), grp / (DB * 4) % KB, grp / 4 % DB, grp % 4, sum);
     }
     parts += GB * C::THREADS;
+  }
+}
+
+// ============================================================================
+// dK / dV of sink keys
+// ============================================================================
+// With sink keys and a bounded window, key j < n_sink is seen by every later row of its
+// sequence: a few keys against all the rows, far too thin for MFMA tiles.  Left to the dK/dV
+// kernel, the first key tile of every sequence walked every query tile with one wave of four
+// at work and took several times as long as any other block (a pack of 65536 tokens in four
+// sequences: 10.8 ms, a third of it that tail).  So the dK/dV kernel treats sink keys like any
+// other key (band pairs only), and this kernel, which runs after it, computes the sink keys'
+// complete dK / dV -- all the rows that see them, inside the window and beyond -- as plain
+// fp32 vector work at memory speed, and overwrites those few rows of dk / dv:
+//   s = q . k_j, P = exp2(s c - lse2), dP = dO . v_j, dS = P (dP - delta)
+//   dV_j = sum P dO, dK_j = scale sum dS q
+// One block per (sequence, kv head, chunk of rows); Q and dO are read once per pass of kSinkPass
+// sink keys; a lane owns 8 consecutive d of one row at a time (D / 8 lanes per row), the dot
+// products are summed across those lanes, and the block's sums -- added in a fixed order -- go
+// to the workspace as fp32 [unit][chunk][sink][dK, dV][D].  The block of a unit that arrives
+// last adds the chunks in chunk order and writes the rows (same protocol as the split dK/dV
+// blocks: deterministic, nobody waits).
+constexpr int kSinkPass = 4;
+
+// sum over the aligned group of W = 8 or 16 lanes, in every lane of the group
+template <int W>
+__device__ __forceinline__ float lane_group_sum(float x) {
+  auto dpp = [](float v, auto ctrl) __attribute__((always_inline)) {
+    return __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), decltype(ctrl)::value,
+                                                       0xf, 0xf, true));
+  };
+  if constexpr (W == 16) x += dpp(x, std::integral_constant<int, 0x140>{});  // row_mirror
+  x += dpp(x, std::integral_constant<int, 0x141>{});                          // row_half_mirror
+  x += dpp(x, std::integral_constant<int, 0x1b>{});                           // quad_perm 3 2 1 0
+  x += dpp(x, std::integral_constant<int, 0xb1>{});                           // quad_perm 1 0 3 2
+  return x;
+}
+
+template <typename T, int D>
+__global__ __launch_bounds__(256) void attn_bwd_sink_kernel(const AttnArgs a) {
+  using V8 = typename Mma<T>::V8;
+  constexpr int LPR = D / 8;     // lanes per row
+  constexpr int RPW = 64 / LPR;  // rows per wave pass
+  constexpr int NS = kSinkPass;
+  constexpr int NSRC = 4 * RPW;  // (wave, row group) sources of the block's sums
+  __shared__ float red_s[NSRC][NS * 2 * D];
+  static_assert(sizeof(red_s) <= 65536, "staging buffer");
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int sub = lane % LPR, rg = lane / LPR;
+  const int c = blockIdx.x % a.sink_chunks;
+  const int unit = blockIdx.x / a.sink_chunks;  // (sequence, kv head)
+  const int hk = unit % a.heads_kv, b = unit / a.heads_kv;
+  int64_t q_row0 = 0, k_row0 = 0;
+  int len_q = a.seqlen_q, len_k = a.seqlen_k;
+  if (a.cu_q) {
+    q_row0 = a.cu_q[b];
+    k_row0 = a.cu_k[b];
+    len_q = a.cu_q[b + 1] - a.cu_q[b];
+    len_k = a.cu_k[b + 1] - a.cu_k[b];
+  }
+  const int ns_all = min(a.n_sink, len_k);
+  // rows of the sequence in n_chunks chunks (at most a.sink_chunks)
+  const int rows_per = (len_q + a.sink_chunks - 1) / a.sink_chunks;
+  const int n_chunks = rows_per > 0 ? (len_q + rows_per - 1) / rows_per : 0;
+  if (c >= n_chunks || ns_all == 0) return;
+  const int shift = a.shift_explicit ? a.shift_val : len_k - len_q;
+  const int r_begin = c * rows_per, r_end = min(len_q, r_begin + rows_per);
+
+  const T* q_ptr = (const T*)a.q + b * a.q_st[0] + q_row0 * a.q_st[1];
+  const T* do_ptr = (const T*)a.dout + b * a.do_st[0] + q_row0 * a.do_st[1];
+  const T* k_ptr = (const T*)a.k + b * a.k_st[0] + k_row0 * a.k_st[1] + hk * a.k_st[2];
+  const T* v_ptr = (const T*)a.v + b * a.v_st[0] + k_row0 * a.v_st[1] + hk * a.v_st[2];
+  const int64_t ws_row0 = a.cu_q ? q_row0 : (int64_t)b * a.seqlen_q;
+  float* out = a.sink_part + ((int64_t)unit * a.sink_chunks + c) * (a.n_sink * 2 * D);
+
+  for (int j0 = 0; j0 < ns_all; j0 += NS) {
+    float kf[NS][8], vf[NS][8], acck[NS][8], accv[NS][8];
+#pragma unroll
+    for (int jj = 0; jj < NS; jj++) {
+      V8 k8 = V8{0, 0, 0, 0, 0, 0, 0, 0}, v8 = k8;
+      if (j0 + jj < ns_all) {
+        k8 = *(const V8*)(k_ptr + (int64_t)(j0 + jj) * a.k_st[1] + sub * 8);
+        v8 = *(const V8*)(v_ptr + (int64_t)(j0 + jj) * a.v_st[1] + sub * 8);
+      }
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        kf[jj][e] = (float)k8[e];
+        vf[jj][e] = (float)v8[e];
+        acck[jj][e] = 0.f;
+        accv[jj][e] = 0.f;
+      }
+    }
+    for (int h = 0; h < a.group; h++) {
+      const int hq = hk * a.group + h;
+      const T* qh = q_ptr + (int64_t)hq * a.q_st[2] + sub * 8;
+      const T* doh = do_ptr + (int64_t)hq * a.do_st[2] + sub * 8;
+      const float* lse_h = a.lse2 + (int64_t)hq * a.rows_q + ws_row0;
+      const float* delta_h = a.delta + (int64_t)hq * a.rows_q + ws_row0;
+      for (int base = r_begin + wave * RPW; base < r_end; base += 4 * RPW) {
+        const int row = base + rg;
+        const bool valid = row < r_end;
+        V8 q8 = V8{0, 0, 0, 0, 0, 0, 0, 0}, d8 = q8;
+        float nl = -__builtin_inff(), nd = 0.f;  // the statistics are stored negated
+        if (valid) {
+          q8 = *(const V8*)(qh + (int64_t)row * a.q_st[1]);
+          d8 = *(const V8*)(doh + (int64_t)row * a.do_st[1]);
+          nl = lse_h[row];
+          nd = delta_h[row];
+        }
+        float qf[8], df[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          qf[e] = (float)q8[e];
+          df[e] = (float)d8[e];
+        }
+        const int hi = (a.wr >= 0) ? min(len_k - 1, row + shift + a.wr) : len_k - 1;
+#pragma unroll
+        for (int jj = 0; jj < NS; jj++) {
+          float sdot = 0.f, pdot = 0.f;
+#pragma unroll
+          for (int e = 0; e < 8; e++) {
+            sdot = __builtin_fmaf(qf[e], kf[jj][e], sdot);
+            pdot = __builtin_fmaf(df[e], vf[jj][e], pdot);
+          }
+          sdot = lane_group_sum<LPR>(sdot);
+          pdot = lane_group_sum<LPR>(pdot);
+          const int j = j0 + jj;
+          const bool vis = valid && j < ns_all && j <= hi;  // a sink key: no lower bound
+          const float p = vis ? __builtin_amdgcn_exp2f(__builtin_fmaf(sdot, a.scale_log2, nl)) : 0.f;
+          const float ds = vis ? p * (pdot + nd) : 0.f;
+#pragma unroll
+          for (int e = 0; e < 8; e++) {
+            accv[jj][e] = __builtin_fmaf(p, df[e], accv[jj][e]);
+            acck[jj][e] = __builtin_fmaf(ds, qf[e], acck[jj][e]);
+          }
+        }
+      }
+    }
+    // the block's sums: every (wave, row group) source staged, then added in source order
+    __syncthreads();  // the previous pass's readers are done
+#pragma unroll
+    for (int jj = 0; jj < NS; jj++)
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        red_s[wave * RPW + rg][(jj * 2 + 0) * D + sub * 8 + e] = acck[jj][e];
+        red_s[wave * RPW + rg][(jj * 2 + 1) * D + sub * 8 + e] = accv[jj][e];
+      }
+    __syncthreads();
+    for (int idx = tid; idx < NS * 2 * D; idx += 256) {
+      float sum = 0.f;
+#pragma unroll
+      for (int src = 0; src < NSRC; src++) sum += red_s[src][idx];
+      const int jj = idx / (2 * D);
+      if (j0 + jj < ns_all) out[(int64_t)(j0 + jj) * (2 * D) + idx % (2 * D)] = sum;
+    }
+  }
+  // count this chunk in; the last one of the unit adds them all up
+  __shared__ int arrived_s;
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  if (tid == 0) {
+    __threadfence();
+    arrived_s = atomicAdd(a.sink_count + unit, 1);
+  }
+  __syncthreads();
+  if (arrived_s != n_chunks - 1) return;
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+  if (tid == 0) a.sink_count[unit] = 0;  // the next launch on this workspace starts from zero
+  T* dk_ptr = (T*)a.dk + b * a.dk_st[0] + k_row0 * a.dk_st[1] + hk * a.dk_st[2];
+  T* dv_ptr = (T*)a.dv + b * a.dv_st[0] + k_row0 * a.dv_st[1] + hk * a.dv_st[2];
+  const float* parts = a.sink_part + (int64_t)unit * a.sink_chunks * (a.n_sink * 2 * D);
+  for (int idx = tid; idx < ns_all * 2 * D; idx += 256) {
+    float sum = 0.f;
+    for (int cc = 0; cc < n_chunks; cc++) sum += parts[(int64_t)cc * (a.n_sink * 2 * D) + idx];
+    const int j = idx / (2 * D), dd = idx % D;
+    if ((idx / D) & 1) {
+      dv_ptr[(int64_t)j * a.dv_st[1] + dd] = (T)sum;
+    } else {
+      dk_ptr[(int64_t)j * a.dk_st[1] + dd] = (T)(sum * a.scale);
+    }
   }
 }
 
@@ -899,6 +1079,7 @@ __global__ __launch_bounds__(256) void attn_bwd_prep_kernel(const AttnArgs a) {
   template __global__ void attn_bwd_dkdv_kernel<T, D, true, true>(const AttnArgs);   \
   template __global__ void attn_bwd_dq_kernel<T, D, false>(const AttnArgs);          \
   template __global__ void attn_bwd_dq_kernel<T, D, true>(const AttnArgs);           \
+  template __global__ void attn_bwd_sink_kernel<T, D>(const AttnArgs);                  \
   template __global__ void attn_bwd_prep_kernel<T, D>(const AttnArgs);
 RSWA_INSTANTIATE(__bf16, 128)
 RSWA_INSTANTIATE(__bf16, 64)
@@ -937,6 +1118,13 @@ int launch_bwd(AttnArgs& a, hipStream_t stream, int phases) {
         else hipLaunchKernelGGL((attn_bwd_dkdv_kernel<T, D, false, false>), grid, block, 0, stream, a);
       }
       int rc = check_launch("attn_bwd dkdv");
+      if (rc != RSWA_OK) return rc;
+    }
+    if (a.n_work > 0 && a.sink_part && a.rows_q > 0) {
+      clear_launch_error();
+      hipLaunchKernelGGL((attn_bwd_sink_kernel<T, D>), dim3(a.batch * a.heads_kv * a.sink_chunks),
+                         dim3(256), 0, stream, a);
+      int rc = check_launch("attn_bwd sink");
       if (rc != RSWA_OK) return rc;
     }
   }

@@ -56,6 +56,12 @@ struct AttnArgs {
   // tiles (forward, dQ) or key tiles (dK/dV) so that the tiles with the most visible
   // pairs start first and the short ones fill the tail of the launch.
   int32_t rev_q, rev_k;
+  // backward with sink keys and a bounded window: workspace of the sink kernel -- fp32 sums
+  // [sequence x kv head][chunk of rows][sink][dK, dV][D] and one arrival counter per
+  // (sequence, kv head); null when that kernel does not run
+  float* sink_part;
+  int32_t* sink_count;
+  int32_t sink_chunks;  // row chunks per (sequence, kv head)
   int32_t far;  // a sequence of some streamed tensor spans 2 GiB or more: FAR kernels
   float scale, scale_log2;
 };
@@ -412,6 +418,9 @@ struct BwdLayout {
   int n_tile_k;            // key tile slots per kv head (dense: per batch entry)
   int n_count;             // arrival counters (one per key tile unit)
   uint64_t count_off, part_off, total_bytes;
+  int sink_chunks;         // row chunks of the sink kernel per (sequence, kv head); 0: no sink kernel
+  int sink_count_index;    // its first arrival counter
+  uint64_t sink_off;       // its fp32 sums
 };
 BwdLayout bwd_layout(const rswa_attn_params* p, bool allow_split);
 

@@ -50,6 +50,16 @@ DENSE_CASES = [
     (1, 513, 513, 2, 2, 128, (1000, 0), True, 2),
     (1, 2048, 2048, 4, 2, 128, (500, 0), True, 0),
     (1, 1, 1, 1, 1, 128, (5, 0), True, 0),
+    # sink keys under a bounded window: their dK / dV rows come from the sink kernel, in
+    # passes of four keys -- one pass partly filled, several passes, sinks across two key tiles,
+    # more sinks than keys, queries aligned to the end of a longer key range, two-sided window
+    (1, 900, 900, 4, 2, 128, (64, 0), True, 3),
+    (1, 1200, 1200, 6, 2, 64, (100, 0), True, 9),
+    (2, 1500, 1500, 2, 1, 128, (32, 0), True, 70),
+    (1, 1100, 1100, 4, 4, 64, (16, 0), True, 300),
+    (1, 40, 40, 2, 1, 128, (3, 0), True, 64),
+    (1, 300, 800, 4, 2, 128, (50, 0), True, 5),
+    (1, 600, 600, 2, 2, 64, (30, 20), False, 6),
 ]
 
 
@@ -155,6 +165,7 @@ def test_bwd_into_strided_views():
     ([5, 130, 64, 1, 300], (50, 0), 0),
     ([257, 255], (-1, 0), 0),
     ([100, 400, 129], (64, 0), 4),
+    ([3, 700, 1, 260, 2000], (40, 0), 7),
 ])
 def test_bwd_varlen_matches_oracle(lens, window, ns):
     from ring_swa.ops import wrapped_flash_attn_bwd_varlen, wrapped_flash_attn_fwd_varlen
