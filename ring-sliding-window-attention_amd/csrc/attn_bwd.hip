@@ -22,7 +22,9 @@
 // DKDV per (query tile, wave) (C layout: lane = key; two 32-key blocks per wave, so every
 // fragment read from LDS feeds two MFMAs):
 //   S = Q K^T, dP = dO V^T      A = Q / dO row fragments (LDS), B = K (registers) / V (LDS)
-//   P = exp2(S*c - lse2), dS = P * (dP - delta); the dP chains start from -delta instead of zero
+//   P = exp2(S*c - lse2), dS = P * (dP - delta): K is multiplied by c when it is loaded, the S
+//   chains start from -lse2 and the dP chains from -delta instead of zero, so one exponential,
+//   one product and the two 16-bit conversions are all the vector work per score
 //   dV^T += dO^T P, dK^T += Q^T dS   A = transposing LDS reads of dO / Q, B = P / dS (regs)
 // The S and dP MFMAs are inline assembly so that their accumulators live in vector
 // registers, where the vector ALU reads them next; left to the compiler they end up in
@@ -147,7 +149,9 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   const int t_row1 = (rl + 8) * C::ROWB + ((lp ^ swz_f<C::CPR>(rl + 8)) << 4) + (i16 & 1) * 8;
 
   // ---- this wave's K fragments stay in registers for the whole walk (B operand of
-  // S = Q K^T: lane = key column, 8 consecutive d per k-step); keys past the end are zero
+  // S = Q K^T: lane = key column, 8 consecutive d per k-step), multiplied by the softmax scale
+  // in base-2 units once here, so that the S chains yield the exponent directly; keys past the
+  // end are zero
   V8 kf[KB][KS];
 #pragma unroll
   for (int kb = 0; kb < KB; kb++) {
@@ -155,7 +159,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
       if (jc < len_k) {
-        kf[kb][ks] = *(const V8*)(k_ptr + (int64_t)jc * a.k_st[1] + ks * 16 + g * 8);
+        const V8 raw = *(const V8*)(k_ptr + (int64_t)jc * a.k_st[1] + ks * 16 + g * 8);
+        float scaled[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) scaled[j] = (float)raw[j] * a.scale_log2;
+        kf[kb][ks] = M::pack(scaled);
       } else {
         kf[kb][ks] = V8{0, 0, 0, 0, 0, 0, 0, 0};
       }
@@ -330,7 +338,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
       };
       f32x16 sacc[KB], pacc[KB];
       f32x16 dinit;  // -delta of the 32 rows in the accumulator layout: the dP chains start from it
-      f32x4 l4[4];   // -lse2 of the rows
+      f32x16 linit;  // -lse2 of the rows, likewise: the S chains start from it
       V8 pb[KB][2], dsb[KB][2];
       // vector work in 2 KB chunks of four rows: chunk order lets the packed operands of
       // the first k-step be complete first
@@ -347,7 +355,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
 #pragma unroll
         for (int e = 0; e < 4; e++) {
           const int i = 4 * i4 + e;
-          pk[kb][i] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][i], a.scale_log2, l4[i4][e]));
+          pk[kb][i] = __builtin_amdgcn_exp2f(sacc[kb][i]);
         }
         if (!full) {
           // key position relative to the aligned diagonal of row i0: rel(r) = rel0 - r
@@ -377,6 +385,12 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
         if (i4 & 1) dsb[kb][i4 >> 1] = M::pack(dsk[kb]);
       };
 
+#pragma unroll
+      for (int i4 = 0; i4 < 4; i4++) {
+        const f32x4 t4 = *(const f32x4*)(lse_lds + 8 * i4 + 4 * g);
+#pragma unroll
+        for (int e = 0; e < 4; e++) linit[4 * i4 + e] = t4[e];
+      }
       static_for<AH>([&](auto fc) __attribute__((always_inline)) { fetch(fc); });
       fence();
       static_for<4 * NG>([&](auto mc) __attribute__((always_inline)) {
@@ -384,16 +398,16 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
         constexpr int f = m / KB, kb = m % KB;  // fragment slot and key block of this MFMA
         if constexpr (kb == 0) fetch(std::integral_constant<int, f + AH>{});
         if (m < NPART && has_next) load_part(m, qn, don, stn);
-        // row statistics: -delta early in S (the dP chains start from it), -lse2 at its end
+        // row statistics: -delta early in S (the dP chains start from it); -lse2 was read
+        // before the first MFMA, whose chain starts from it
         if constexpr (m >= 4 && m < 8) {
           const f32x4 t4 = *(const f32x4*)(delta_lds + 8 * (m - 4) + 4 * g);
 #pragma unroll
           for (int e = 0; e < 4; e++) dinit[4 * (m - 4) + e] = t4[e];
         }
-        if constexpr (m >= NG - 4 && m < NG) l4[m - (NG - 4)] = *(const f32x4*)(lse_lds + 8 * (m - (NG - 4)) + 4 * g);
         if constexpr (m < NG) {
           if constexpr (f == 0) {
-            M::mfma32_vec0(fa[f], kf[kb][f], sacc[kb]);
+            M::mfma32_vec_init(fa[f], kf[kb][f], linit, sacc[kb]);
           } else {
             M::mfma32_vec(fa[f], kf[kb][f], sacc[kb]);
           }
