@@ -167,6 +167,14 @@ typedef struct rswa_attn_params {
    * one row stride must stay below 8 MiB.  RSWA_ADDR_FAR (1) selects the second form whatever
    * the sizes (same results; a few per cent slower). */
   int32_t addressing;
+  /* Forward only.  != 0: out / lse already hold a running partial result for these rows (16-bit
+   * out, fp32 lse, e.g. what an earlier rswa_attn_fwd over other keys wrote); this call's block is
+   * merged into them in place instead of overwriting them -- the arithmetic of
+   * rswa_merge_attn_out (ring_swa/ops/merge.py:16-50) applied to the block's 16-bit output, in
+   * the kernel's epilogue: same bits as the two calls, one launch and one pass over out less
+   * (what ring_swa/ops/attn.py:23-37 does with a temporary and a merge kernel). */
+  int32_t out_accumulate;
+  int32_t reserved_;
 } rswa_attn_params;
 
 #define RSWA_ADDR_AUTO 0

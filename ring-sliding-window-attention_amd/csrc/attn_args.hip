@@ -156,6 +156,7 @@ int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a, bool allow_
   a.shift_explicit = p->shift_explicit != 0;
   a.shift_val = p->shift;
   a.dq_accumulate = backward && p->dq_accumulate != 0;
+  a.out_accumulate = !backward && p->out_accumulate != 0;
   a.n_tile = 0;
   a.n_work = 0;
   {

@@ -22,9 +22,11 @@
 // DKDV per (query tile, wave) (C layout: lane = key; two 32-key blocks per wave, so every
 // fragment read from LDS feeds two MFMAs):
 //   S = Q K^T, dP = dO V^T      A = Q / dO row fragments (LDS), B = K (registers) / V (LDS)
-//   P = exp2(S*c - lse2), dS = P * (dP - delta): K is multiplied by c when it is loaded, the S
-//   chains start from -lse2 and the dP chains from -delta instead of zero, so one exponential,
-//   one product and the two 16-bit conversions are all the vector work per score
+//   P = exp2(S*c - lse2), dS = P * (dP - delta); the dP chains start from -delta instead of zero.
+//   (Folding c into 16-bit K fragments and starting the S chains from -lse2 would save the
+//   multiply-add per score -- 1-2 % -- but the rounding of K c shifts the exponent by up to
+//   2^-9 |S c|: with peaked scores, e.g. sink keys four times the usual size, it doubled the
+//   error of dK / dV against the fp32 oracle, 4e-3 -> 7e-3.  The scale stays in fp32.)
 //   dV^T += dO^T P, dK^T += Q^T dS   A = transposing LDS reads of dO / Q, B = P / dS (regs)
 // The S and dP MFMAs are inline assembly so that their accumulators live in vector
 // registers, where the vector ALU reads them next; left to the compiler they end up in
@@ -35,9 +37,9 @@
 // registers), so every copy or read the compiler adds around them is padded as required.
 // DQ per (key tile, wave), on 16x16x32 MFMAs; wave owns 32 query columns (lane = query l % 16
 // of two 16-query blocks):
-//   S^T = K Q^T, dP^T = V dO^T  A = K / V row fragments from LDS, B = Q c / dO fragments (regs);
-//                               the chains start from -lse2 / -delta of the lane's queries
-//   dS^T = exp2(S^T) dP^T       (one exponential, one product, the 16-bit conversion per score)
+//   S^T = K Q^T, dP^T = V dO^T  A = K / V row fragments from LDS, B = Q / dO fragments (regs);
+//                               the dP^T chains start from -delta of the lane's queries
+//   dS^T = exp2(S^T c - lse2) dP^T   (the scale is applied in fp32: see the note at DKDV)
 //   dQ^T += K^T dS^T            A = transposing LDS reads of K, B = dS^T (regs)
 //
 // Streamed tiles are double-buffered in SEPARATE static __shared__ arrays, filled by buffer
@@ -149,9 +151,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   const int t_row1 = (rl + 8) * C::ROWB + ((lp ^ swz_f<C::CPR>(rl + 8)) << 4) + (i16 & 1) * 8;
 
   // ---- this wave's K fragments stay in registers for the whole walk (B operand of
-  // S = Q K^T: lane = key column, 8 consecutive d per k-step), multiplied by the softmax scale
-  // in base-2 units once here, so that the S chains yield the exponent directly; keys past the
-  // end are zero
+  // S = Q K^T: lane = key column, 8 consecutive d per k-step); keys past the end are zero
   V8 kf[KB][KS];
 #pragma unroll
   for (int kb = 0; kb < KB; kb++) {
@@ -159,11 +159,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
       if (jc < len_k) {
-        const V8 raw = *(const V8*)(k_ptr + (int64_t)jc * a.k_st[1] + ks * 16 + g * 8);
-        float scaled[8];
-#pragma unroll
-        for (int j = 0; j < 8; j++) scaled[j] = (float)raw[j] * a.scale_log2;
-        kf[kb][ks] = M::pack(scaled);
+        kf[kb][ks] = *(const V8*)(k_ptr + (int64_t)jc * a.k_st[1] + ks * 16 + g * 8);
       } else {
         kf[kb][ks] = V8{0, 0, 0, 0, 0, 0, 0, 0};
       }
@@ -338,7 +334,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
       };
       f32x16 sacc[KB], pacc[KB];
       f32x16 dinit;  // -delta of the 32 rows in the accumulator layout: the dP chains start from it
-      f32x16 linit;  // -lse2 of the rows, likewise: the S chains start from it
+      f32x4 l4[4];   // -lse2 of the rows
       V8 pb[KB][2], dsb[KB][2];
       // vector work in 2 KB chunks of four rows: chunk order lets the packed operands of
       // the first k-step be complete first
@@ -355,7 +351,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
 #pragma unroll
         for (int e = 0; e < 4; e++) {
           const int i = 4 * i4 + e;
-          pk[kb][i] = __builtin_amdgcn_exp2f(sacc[kb][i]);
+          pk[kb][i] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][i], a.scale_log2, l4[i4][e]));
         }
         if (!full) {
           // key position relative to the aligned diagonal of row i0: rel(r) = rel0 - r
@@ -385,12 +381,6 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
         if (i4 & 1) dsb[kb][i4 >> 1] = M::pack(dsk[kb]);
       };
 
-#pragma unroll
-      for (int i4 = 0; i4 < 4; i4++) {
-        const f32x4 t4 = *(const f32x4*)(lse_lds + 8 * i4 + 4 * g);
-#pragma unroll
-        for (int e = 0; e < 4; e++) linit[4 * i4 + e] = t4[e];
-      }
       static_for<AH>([&](auto fc) __attribute__((always_inline)) { fetch(fc); });
       fence();
       static_for<4 * NG>([&](auto mc) __attribute__((always_inline)) {
@@ -398,16 +388,16 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
         constexpr int f = m / KB, kb = m % KB;  // fragment slot and key block of this MFMA
         if constexpr (kb == 0) fetch(std::integral_constant<int, f + AH>{});
         if (m < NPART && has_next) load_part(m, qn, don, stn);
-        // row statistics: -delta early in S (the dP chains start from it); -lse2 was read
-        // before the first MFMA, whose chain starts from it
+        // row statistics: -delta early in S (the dP chains start from it), -lse2 at its end
         if constexpr (m >= 4 && m < 8) {
           const f32x4 t4 = *(const f32x4*)(delta_lds + 8 * (m - 4) + 4 * g);
 #pragma unroll
           for (int e = 0; e < 4; e++) dinit[4 * (m - 4) + e] = t4[e];
         }
+        if constexpr (m >= NG - 4 && m < NG) l4[m - (NG - 4)] = *(const f32x4*)(lse_lds + 8 * (m - (NG - 4)) + 4 * g);
         if constexpr (m < NG) {
           if constexpr (f == 0) {
-            M::mfma32_vec_init(fa[f], kf[kb][f], linit, sacc[kb]);
+            M::mfma32_vec0(fa[f], kf[kb][f], sacc[kb]);
           } else {
             M::mfma32_vec(fa[f], kf[kb][f], sacc[kb]);
           }
@@ -711,11 +701,11 @@ __global__ __launch_bounds__(256) void attn_bwd_sink_kernel(const AttnArgs a) {
 // ============================================================================
 // dQ
 // ============================================================================
-// LDS read-ahead of the dQ kernel's two matrix sections, in fragments (measured: 8 / 4 is
-// 2-3 % faster than 6 / 4 and than 12 / 6; the register file, all 256 registers of a lane
-// at head_dim 128, allows no more in the first section once S^T and dP^T are both live)
+// LDS read-ahead of the dQ kernel's two matrix sections, in fragments (measured: 7 / 4 and
+// 6 / 4 are equal, 12 / 6 is 2-3 % slower; 8 / 4 spills at head_dim 128 -- all 256 registers of
+// a lane are in use in the first section once S^T and dP^T are both live -- and is 5 % slower)
 #ifndef RSWA_DQ_AH1
-#define RSWA_DQ_AH1 8
+#define RSWA_DQ_AH1 7
 #endif
 #ifndef RSWA_DQ_AH2
 #define RSWA_DQ_AH2 4
@@ -820,7 +810,8 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(const AttnArgs a) {
   // conversion per score.  Rounding the scaled Q to 16 bits moves a score by about 2^-9 of its
   // typical magnitude (P by about 0.1 %), a quarter of what rounding P itself to 16 bits does.
   V8 qf[2][KS], dof[2][KS];
-  f32x4 lse2[2], delta[2];  // the row's value in all four elements
+  float lse2[2];   // -lse2 of the lane's two queries
+  f32x4 delta[2];  // -delta of the same, in all four elements (start value of the dP^T chains)
 #pragma unroll
   for (int qb = 0; qb < 2; qb++) {
     const int iq = r0 + 16 * qb + r;
@@ -828,11 +819,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(const AttnArgs a) {
     if (iq < len_q) {
 #pragma unroll
       for (int ks = 0; ks < KS; ks++) {
-        const V8 qraw = *(const V8*)(q_ptr + (int64_t)iq * a.q_st[1] + ks * 32 + u * 8);
-        float qs[8];
-#pragma unroll
-        for (int j = 0; j < 8; j++) qs[j] = (float)qraw[j] * a.scale_log2;
-        qf[qb][ks] = M::pack(qs);
+        qf[qb][ks] = *(const V8*)(q_ptr + (int64_t)iq * a.q_st[1] + ks * 32 + u * 8);
         dof[qb][ks] = *(const V8*)(do_ptr + (int64_t)iq * a.do_st[1] + ks * 32 + u * 8);
       }
       l2 = a.lse2[(int64_t)hq * a.rows_q + ws_row0 + iq];
@@ -844,7 +831,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(const AttnArgs a) {
         dof[qb][ks] = V8{0, 0, 0, 0, 0, 0, 0, 0};
       }
     }
-    lse2[qb] = f32x4{l2, l2, l2, l2};
+    lse2[qb] = l2;
     delta[qb] = f32x4{dl, dl, dl, dl};
   }
 
@@ -903,7 +890,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(const AttnArgs a) {
           const V8 vfrag = *(const V8*)(vc + off);
 #pragma unroll
           for (int qb = 0; qb < 2; qb++) {
-            sacc[kb][qb] = M::mfma16(kfrag, qf[qb][ks], ks == 0 ? lse2[qb] : sacc[kb][qb]);
+            sacc[kb][qb] = M::mfma16(kfrag, qf[qb][ks], ks == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : sacc[kb][qb]);
             pacc[kb][qb] = M::mfma16(vfrag, dof[qb][ks], ks == 0 ? delta[qb] : pacc[kb][qb]);
           }
         }
@@ -945,7 +932,8 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(const AttnArgs a) {
 #pragma unroll
             for (int e = 0; e < 8; e++) {
               const int kb = 2 * ks2 + (e >> 2), i = e & 3;
-              float ds = __builtin_amdgcn_exp2f(sacc[kb][qb][i]) * pacc[kb][qb][i];
+              float ds = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][qb][i], a.scale_log2, lse2[qb])) *
+                         pacc[kb][qb][i];
               if constexpr (!FULL) {
                 const int j = 16 * kb + 4 * u_m + i;
                 const bool ok = (j <= hi_rel[qb]) & ((j >= lo_rel[qb]) | (j < sink_rel));

@@ -50,6 +50,7 @@ struct AttnArgs {
   int32_t wl, wr, n_sink;  // wl/wr < 0: unbounded
   int32_t shift_explicit, shift_val;
   int32_t dq_accumulate;  // backward: add to dq instead of overwriting it
+  int32_t out_accumulate;  // forward: merge the block into what out / lse hold
   int32_t n_tile;          // tiles per sequence (dense) / total tile slots (packed)
   int32_t n_work;          // logical blocks
   // Blocks are dispatched in logical order; these flags reverse the order of the query

@@ -334,37 +334,71 @@ __global__ __launch_bounds__(512) void attn_fwd_kernel(const AttnArgs a) {
   // ---- epilogue --------------------------------------------------------------
   const float l_tot = halfwave_sum(l_run);
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-  if (g == 0 && iq < len_q) {
-    lse_ptr[(int64_t)iq * a.lse_st[2]] =
-        l_tot > 0.f ? m_run * a.scale + __logf(l_tot) : -__builtin_inff();
-  }
   // transpose O^T through LDS for coalesced 16-byte stores: waves 0-3 first (one tile
   // buffer each), then waves 4-7
   char* stage = (wave & 3) == 0 ? k_s0 : (wave & 3) == 1 ? k_s1 : (wave & 3) == 2 ? v_s0 : v_s1;
-  for (int half = 0; half < 2; half++) {
-    if ((wave >> 2) == half) {
-#pragma unroll
-      for (int d = 0; d < C::DBLK; d++)
-#pragma unroll
-        for (int i4 = 0; i4 < 4; i4++) {
-          const auto h4 = M::pack4(o_acc[d][4 * i4] * inv, o_acc[d][4 * i4 + 1] * inv,
-                                   o_acc[d][4 * i4 + 2] * inv, o_acc[d][4 * i4 + 3] * inv);
-          *(typename M::V4*)(stage + l32 * C::O_STRIDE + (d * 32 + 8 * i4 + 4 * g) * 2) = h4;
-        }
+  // out_accumulate: out / lse hold a running partial result; the block is merged into it with
+  // the arithmetic of the merge kernel (merge_lse.hip), applied to the block's output after
+  // its rounding to 16 bits -- the same bits as a forward into a temporary plus a merge.  The
+  // rows' two weights wait in LDS behind the staged tile for the lanes that store the rows.
+  float* wgt = (float*)(stage + 32 * C::O_STRIDE);
+  static_assert(C::TILE >= 32 * C::O_STRIDE + 32 * 2 * 4, "weights fit behind the staged tile");
+  {
+    const float ninf = -__builtin_inff();
+    float lse_new = l_tot > 0.f ? m_run * a.scale + __logf(l_tot) : ninf;
+    float w_old = 0.f, w_new = 1.f;
+    if (a.out_accumulate && iq < len_q) {
+      const float la = lse_ptr[(int64_t)iq * a.lse_st[2]], lb = lse_new;
+      const bool both_empty = (la == ninf) && (lb == ninf);
+      const float diff = both_empty ? 0.f : lb - la;
+      w_old = both_empty ? 0.f : 1.f / (1.f + __expf(diff));
+      w_new = both_empty ? 0.f : 1.f / (1.f + __expf(-diff));
+      lse_new = both_empty ? ninf : fmaxf(la, lb) + log1pf(__expf(-fabsf(diff)));
     }
-    __syncthreads();
-    if ((wave >> 2) == half) {
+    if (g == 0 && iq < len_q) lse_ptr[(int64_t)iq * a.lse_st[2]] = lse_new;
+    for (int half = 0; half < 2; half++) {
+      if ((wave >> 2) == half) {
 #pragma unroll
-      for (int n = 0; n < 32 * C::CPR / 64; n++) {
-        const int c = lane + n * 64;
-        const int row = c / C::CPR, col = (c % C::CPR) * 8;
-        if (r0 + row < len_q) {
-          const u32x4 val = *(const u32x4*)(stage + row * C::O_STRIDE + col * 2);
-          *(u32x4*)(o_ptr + (int64_t)(r0 + row) * a.o_st[1] + col) = val;
+        for (int d = 0; d < C::DBLK; d++)
+#pragma unroll
+          for (int i4 = 0; i4 < 4; i4++) {
+            const auto h4 = M::pack4(o_acc[d][4 * i4] * inv, o_acc[d][4 * i4 + 1] * inv,
+                                     o_acc[d][4 * i4 + 2] * inv, o_acc[d][4 * i4 + 3] * inv);
+            *(typename M::V4*)(stage + l32 * C::O_STRIDE + (d * 32 + 8 * i4 + 4 * g) * 2) = h4;
+          }
+        if (g == 0) {
+          wgt[2 * l32] = w_old;
+          wgt[2 * l32 + 1] = w_new;
         }
       }
+      __syncthreads();
+      if ((wave >> 2) == half) {
+#pragma unroll
+        for (int n = 0; n < 32 * C::CPR / 64; n++) {
+          const int c = lane + n * 64;
+          const int row = c / C::CPR, col = (c % C::CPR) * 8;
+          if (r0 + row < len_q) {
+            V8 val = *(const V8*)(stage + row * C::O_STRIDE + col * 2);
+            T* dst = o_ptr + (int64_t)(r0 + row) * a.o_st[1] + col;
+            if (a.out_accumulate) {
+              const float wo = wgt[2 * row], wn = wgt[2 * row + 1];
+              const V8 old = *(const V8*)dst;
+              float y[8];
+#pragma unroll
+              for (int j = 0; j < 8; j++) {
+                // a zero weight must annihilate whatever the other side holds
+                const float t0 = (wo == 0.f) ? 0.f : (float)old[j] * wo;
+                const float t1 = (wn == 0.f) ? 0.f : (float)val[j] * wn;
+                y[j] = t0 + t1;
+              }
+              val = M::pack(y);
+            }
+            *(V8*)dst = val;
+          }
+        }
+      }
+      __syncthreads();
     }
-    __syncthreads();
   }
 }
 

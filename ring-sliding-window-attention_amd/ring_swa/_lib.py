@@ -72,6 +72,8 @@ class AttnParams(Structure):
         ("workspace_bytes", c_uint64),
         ("dq_accumulate", c_int32),
         ("addressing", c_int32),
+        ("out_accumulate", c_int32),
+        ("reserved_", c_int32),
     ]
 
 

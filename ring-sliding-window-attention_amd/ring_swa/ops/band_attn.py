@@ -111,31 +111,48 @@ def attn_fwd(
     *,
     num_sink: int = 0,
     mask_shift: Optional[int] = None,
+    accumulate_into: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Masked attention forward on the HIP kernel; returns ``(out, lse)``."""
+    """Masked attention forward on the HIP kernel; returns ``(out, lse)``.
+
+    ``accumulate_into=(out, lse)``: running partial results of these rows (``out`` in q's
+    dtype, ``lse`` fp32, views allowed) that this block is merged into in place, in the
+    kernel's epilogue -- the same bits as a forward into temporaries followed by
+    ``merge_attn_out``, without the temporaries and the second pass."""
     packed = cu_seqlens_q is not None
     _check_qkv(q, k, v, packed)
     dev = _lib.require_device(q, k, v)
     if softmax_scale is None:
         softmax_scale = q.shape[-1] ** (-0.5)
-    out = torch.empty(q.shape, dtype=q.dtype, device=dev)
-    if packed:
-        lse = torch.empty((q.shape[1], q.shape[0]), dtype=torch.float32, device=dev)
+    lse_shape = (q.shape[1], q.shape[0]) if packed else (q.shape[0], q.shape[2], q.shape[1])
+    if accumulate_into is not None:
+        out, lse = accumulate_into
+        assert out.shape == q.shape and out.dtype == q.dtype and out.stride(-1) == 1, (
+            "accumulate_into: out must have q's shape and dtype"
+        )
+        assert tuple(lse.shape) == lse_shape and lse.dtype == torch.float32, (
+            "accumulate_into: lse must be fp32 [batch, heads, seq] ([heads, tokens] when packed)"
+        )
+        _lib.require_device(out, lse)
+        if q.numel() == 0 or k.numel() == 0:
+            return out, lse  # an empty block is the identity of the merge
     else:
-        lse = torch.empty((q.shape[0], q.shape[2], q.shape[1]), dtype=torch.float32, device=dev)
-    if q.numel() == 0:
-        return out, lse
-    if k.numel() == 0:
-        # no keys at all: every row is empty (out = 0, lse = -inf), as attn_bwd assumes
-        out.zero_()
-        lse.fill_(float("-inf"))
-        return out, lse
+        out = torch.empty(q.shape, dtype=q.dtype, device=dev)
+        lse = torch.empty(lse_shape, dtype=torch.float32, device=dev)
+        if q.numel() == 0:
+            return out, lse
+        if k.numel() == 0:
+            # no keys at all: every row is empty (out = 0, lse = -inf), as attn_bwd assumes
+            out.zero_()
+            lse.fill_(float("-inf"))
+            return out, lse
     p = _params(q, k, v, softmax_scale, window_size, causal, cu_seqlens_q, cu_seqlens_k, num_sink,
                 mask_shift)
     p.out = out.data_ptr()
     p.out_stride = _lib.i64x3(_strides3(out, packed))
     p.lse = lse.data_ptr()
     p.lse_stride = _lib.i64x3(_lse_strides(lse, packed))
+    p.out_accumulate = 0 if accumulate_into is None else 1
     with torch.cuda.device(dev):
         _lib.check(_lib.lib().rswa_attn_fwd(p, _lib.stream_ptr(dev)))
     return out, lse

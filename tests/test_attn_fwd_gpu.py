@@ -188,3 +188,43 @@ def test_fwd_without_any_key_gives_the_empty_row_pair():
     attn_bwd(q, k, k.clone(), out, lse, torch.ones_like(q), dq, dk, dv, None, (16, 0), True)
     torch.cuda.synchronize()
     assert (dq == 0).all()
+
+
+@pytest.mark.parametrize("case", [
+    # (B, Sq, Sk, Hq, Hkv, D, window, causal, dtype): a second block merged into the result of a first
+    (1, 512, 512, 4, 2, 128, (0, 512), False, torch.bfloat16),    # previous-chunk corner
+    (2, 300, 200, 4, 4, 64, (-1, -1), False, torch.bfloat16),
+    (1, 777, 500, 2, 1, 128, (100, 50), False, torch.float16),    # rows with no key in the block
+    (1, 200, 333, 6, 2, 64, (40, 0), True, torch.bfloat16),
+], ids=["corner", "full", "two_sided_f16", "causal_sq_lt_sk"])
+def test_fwd_accumulate_into_equals_forward_plus_merge(case):
+    """out_accumulate of the ABI: the block merged into running (out, lse) in the forward's
+    epilogue must give the bits of a forward into temporaries followed by the merge kernel;
+    rows that the running result, the block, or both leave empty included."""
+    from ring_swa.ops import attn_fwd, merge_attn_out
+
+    b, sq, sk, hq, hk, d, window, causal, dtype = case
+    torch.manual_seed(9)
+    q = torch.randn(b, sq, hq, d, device="cuda").to(dtype)
+    k1, v1 = (torch.randn(b, sq, hk, d, device="cuda").to(dtype) for _ in range(2))
+    k2, v2 = (torch.randn(b, sk, hk, d, device="cuda").to(dtype) for _ in range(2))
+    # running result: a causal band of width 64 over the first keys -- with sq > 64 ... some
+    # rows are empty only if the mask says so; make the first 5 rows empty on purpose
+    out0, lse0 = attn_fwd(q, k1, v1, None, (64, 0), True)
+    out0[:, :5] = 0
+    lse0[:, :, :5] = float("-inf")
+    ref_out, ref_lse = out0.clone(), lse0.clone()
+    o2, l2 = attn_fwd(q, k2, v2, None, window, causal)
+    merge_attn_out(ref_out, ref_lse, o2, l2)
+    got_out, got_lse = out0.clone(), lse0.clone()
+    r = attn_fwd(q, k2, v2, None, window, causal, accumulate_into=(got_out, got_lse))
+    assert r[0] is got_out and r[1] is got_lse
+    assert torch.equal(got_lse, ref_lse)
+    assert torch.equal(got_out, ref_out)
+    # views: only a row range of a larger running result
+    big_out, big_lse = out0.clone(), lse0.clone()
+    n = sq // 2
+    attn_fwd(q[:, :n], k2, v2, None, window, causal, mask_shift=sk - sq,
+             accumulate_into=(big_out[:, :n], big_lse[:, :, :n]))
+    assert torch.equal(big_out[:, n:], out0[:, n:]) and torch.equal(big_lse[:, :, n:], lse0[:, :, n:])
+    assert torch.equal(big_out[:, :n], ref_out[:, :n]) and torch.equal(big_lse[:, :, :n], ref_lse[:, :, :n])
