@@ -357,8 +357,8 @@ def main():
             "workload": "c3_rank_share",
             "detail": "1 rank of virtual cp 8: chunk 8192 of seq 65536, 32 q / 8 kv heads, "
                       "head_dim 128, window 4096; own-chunk band + previous-chunk corner + LSE "
-                      "merge; fwd+bwd via autograd; ring_dtypes=False: the two blocks' 16-bit outputs and fp32 LSE "
-                      "are merged once; the reference's accumulator types (fp32 output, fp64 "
+                      "merge; fwd+bwd via autograd; ring_dtypes=False: the second block is merged into the "
+                      "first one's 16-bit output and fp32 LSE in its forward launch's epilogue (one rounding); the reference's accumulator types (fp32 output, fp64 "
                       "LSE, one merge per block) are ring_dtypes=True, timed as "
                       "ms_per_step_ring_dtypes",
             "ring_dtypes": False,
