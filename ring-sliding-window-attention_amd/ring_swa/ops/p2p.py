@@ -30,15 +30,40 @@ def get_group_local_to_global_rank_map(group) -> Dict[int, int]:
     return dict(enumerate(dist.get_process_group_ranks(group)))
 
 
+class _StagedWork:
+    """Requests of a batch whose device tensors travel through host memory: ``wait`` completes
+    the transfers and copies what was received into the device buffers."""
+
+    def __init__(self, works, landed):
+        self._works, self._landed = works, landed
+
+    def wait(self):
+        for w in self._works:
+            w.wait()
+        for buf, host in self._landed:
+            buf.copy_(host)
+        self._landed = []
+
+
 def exchange(sends: Sequence[Tuple[torch.Tensor, int]], recvs: Sequence[Tuple[torch.Tensor, int]],
              group) -> List["dist.Work"]:
     """Post every ``(tensor, global destination)`` send and ``(buffer, global source)``
     receive of one phase as a single batch; returns the requests to wait on.  Tensors must be
-    contiguous; an empty phase returns no requests."""
+    contiguous; an empty phase returns no requests.
+
+    A gloo group takes host tensors only: device tensors are staged through host memory
+    (synchronous copy out before the send, copy back in ``wait``) -- the route for rehearsing
+    the ring with several processes on one GPU; RCCL groups get the device tensors as they are."""
+    if not sends and not recvs:
+        return []
+    on_device = any(t.is_cuda for t, _ in list(sends) + list(recvs))
+    if on_device and dist.get_backend(group) == "gloo":
+        landed = [(buf, torch.empty(buf.shape, dtype=buf.dtype)) for buf, _ in recvs]
+        ops = [dist.P2POp(dist.irecv, host, src, group) for (_, host), (_, src) in zip(landed, recvs)]
+        ops += [dist.P2POp(dist.isend, t.cpu(), dst, group) for t, dst in sends]
+        return [_StagedWork(dist.batch_isend_irecv(ops), landed)]
     ops = [dist.P2POp(dist.irecv, buf, src, group) for buf, src in recvs]
     ops += [dist.P2POp(dist.isend, t, dst, group) for t, dst in sends]
-    if not ops:
-        return []
     return dist.batch_isend_irecv(ops)
 
 

@@ -1,0 +1,106 @@
+"""The context-parallel ring (``ring_swa/ring.py``) with the HIP kernels: 2 and 4 processes
+that share the one GPU, exchanging chunks over gloo (device tensors staged through host
+memory by ``ops/p2p.py``).  No xGMI or RCCL is involved; what this covers is everything else
+of a multi-rank run on real kernels -- views and strides of the received key ranges, the fp32 /
+fp64 accumulators through the merge kernel, dKV going back to its owner -- against the
+reference's own invariant: the ranks' outputs and gradients put together equal the single
+call on the whole sequence (itself checked against the oracle elsewhere)."""
+import os
+import socket
+import sys
+
+import pytest
+import torch
+import torch.distributed as dist
+import torch.multiprocessing as mp
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HQ, HK, D = 8, 2, 128
+
+
+def _free_port():
+    with socket.socket() as s:
+        s.bind(("127.0.0.1", 0))
+        return s.getsockname()[1]
+
+
+def _inputs(total, packed, seed):
+    g = torch.Generator().manual_seed(seed)
+    lead = () if packed else (2,)
+    q, do = (torch.randn(*lead, total, HQ, D, generator=g).bfloat16() for _ in range(2))
+    k, v = (torch.randn(*lead, total, HK, D, generator=g).bfloat16() for _ in range(2))
+    return q, k, v, do
+
+
+def _cases(world):
+    s = 384  # tokens per rank: 1.5 forward tiles of 256 rows, 3 of 128
+    total = s * world
+    cases = {}
+    for w in (100, s, s + 70, 3 * s - 1, 10 * total):
+        cases[f"dense_w{w}"] = (total, w, None)
+    cases["packed_w200"] = (total, 200, [0, 5, s - 3, s + 130, total])
+    cases[f"packed_w{2 * s}"] = (total, 2 * s, [0, total - 37, total])
+    return cases
+
+
+def _worker(rank, world, port, cases, results):
+    sys.path.insert(0, ROOT)
+    sys.path.insert(0, os.path.join(ROOT, "ring-sliding-window-attention_amd"))
+    torch.cuda.set_device(0)
+    dist.init_process_group("gloo", init_method=f"tcp://127.0.0.1:{port}", rank=rank,
+                            world_size=world)
+    import ring_swa
+
+    group = dist.new_group(list(range(world)))
+    out = {}
+    for n, (name, (total, w, cu)) in enumerate(cases.items()):
+        q, k, v, do = _inputs(total, cu is not None, n)
+        s = total // world
+        sl = slice(rank * s, (rank + 1) * s)
+        if cu is None:
+            qr, kr, vr = (t[:, sl].cuda().requires_grad_() for t in (q, k, v))
+            o = ring_swa.ring_sliding_window_attn(qr, kr, vr, w, group)
+            o.backward(do[:, sl].cuda())
+        else:
+            qr, kr, vr = (t[sl].cuda().requires_grad_() for t in (q, k, v))
+            cu_dev = torch.tensor(cu, dtype=torch.int32, device="cuda")
+            o = ring_swa.ring_sliding_window_attn_varlen(qr, kr, vr, w, cu_dev, group, world, rank)
+            o.backward(do[sl].cuda())
+        torch.cuda.synchronize()
+        out[name] = tuple(t.detach().float().cpu() for t in (o, qr.grad, kr.grad, vr.grad))
+    results[rank] = out
+    dist.barrier()
+    dist.destroy_process_group()
+
+
+@pytest.mark.parametrize("world", [2, 4])
+def test_ring_ranks_on_one_gpu_equal_the_single_call(world):
+    import ring_swa
+
+    cases = _cases(world)
+    port = _free_port()
+    with mp.Manager() as manager:
+        results = manager.dict()
+        mp.spawn(_worker, args=(world, port, cases, results), nprocs=world, join=True)
+        results = dict(results)
+    for n, (name, (total, w, cu)) in enumerate(cases.items()):
+        q, k, v, do = _inputs(total, cu is not None, n)
+        qg, kg, vg = (t.cuda().requires_grad_() for t in (q, k, v))
+        if cu is None:
+            ref = ring_swa.ring_sliding_window_attn(qg, kg, vg, w)
+            cat = 1
+        else:
+            ref = ring_swa.ring_sliding_window_attn_varlen(
+                qg, kg, vg, w, torch.tensor(cu, dtype=torch.int32, device="cuda"))
+            cat = 0
+        ref.backward(do.cuda())
+        refs = [t.detach().float().cpu() for t in (ref, qg.grad, kg.grad, vg.grad)]
+        for idx, r in enumerate(refs):
+            got = torch.cat([results[rk][name][idx] for rk in range(world)], dim=cat)
+            if idx == 0:
+                assert (got - r).abs().max().item() <= 2e-2, f"{name}: out"
+            else:
+                rel = ((got - r).norm() / r.norm().clamp_min(1e-30)).item()
+                assert rel <= 1e-2, f"{name}[{idx}]: rel-norm {rel}"
