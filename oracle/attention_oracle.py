@@ -49,8 +49,13 @@ def window_allowed(
     causal: bool = False,
     n_sink: int = 0,
     device=None,
+    shift: Optional[int] = None,
 ) -> torch.Tensor:
     """Boolean ``[sq, sk]`` matrix, True where query row i may see key j.
+
+    ``shift`` (default ``sk - sq``): the key that query row 0 is aligned with; an explicit
+    value moves the diagonal of the window rule (the out-of-window sink partial of the split
+    streaming path uses ``-(window + 1)``).
 
     Bottom-right alignment: the last query row is aligned with the last key
     (``test/test_local_swa.py:63-85``).  ``causal`` forces the right extent to 0
@@ -63,7 +68,7 @@ def window_allowed(
         wr = 0
     i = torch.arange(sq, device=device).unsqueeze(1)
     j = torch.arange(sk, device=device).unsqueeze(0)
-    rel = j - i - (sk - sq)
+    rel = j - i - ((sk - sq) if shift is None else shift)
     ok = torch.ones(sq, sk, dtype=torch.bool, device=device)
     if wl >= 0:
         ok &= rel >= -wl
@@ -157,14 +162,15 @@ def masked_attention(
 
 def window_attention(
     q, k, v, softmax_scale=None, window=(-1, -1), causal=False, n_sink=0,
-    compute_dtype=torch.float32,
+    compute_dtype=torch.float32, shift=None,
 ):
     """Dense block with flash-attn window semantics -> ``(out, lse)``.
 
     Restates ``ring_swa/ops/wrap_flash.py:168-200`` (what it returns) through
     the closed form of ``test/test_local_swa.py:51-93``.
     """
-    allowed = window_allowed(q.shape[1], k.shape[1], window, causal, n_sink, device=q.device)
+    allowed = window_allowed(q.shape[1], k.shape[1], window, causal, n_sink, device=q.device,
+                             shift=shift)
     return masked_attention(q, k, v, allowed, softmax_scale, compute_dtype)
 
 

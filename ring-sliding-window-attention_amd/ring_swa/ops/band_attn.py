@@ -250,34 +250,38 @@ def bwd_workspace_bytes(q: torch.Tensor, k: torch.Tensor,
 
 
 # ---- names of the upstream wrappers -----------------------------------------
-def wrapped_flash_attn_fwd(q, k, v, softmax_scale, window_size, causal, *, num_sink=0):
-    """Dense forward, ``ring_swa/ops/wrap_flash.py:168``: returns ``(out, softmax_lse)``."""
-    return attn_fwd(q, k, v, softmax_scale, window_size, causal, num_sink=num_sink)
+def wrapped_flash_attn_fwd(q, k, v, softmax_scale, window_size, causal, *, num_sink=0,
+                           mask_shift=None):
+    """Dense forward, ``ring_swa/ops/wrap_flash.py:168``: returns ``(out, softmax_lse)``.
+    ``mask_shift`` replaces the bottom-right alignment ``len_k - len_q`` of the window rule."""
+    return attn_fwd(q, k, v, softmax_scale, window_size, causal, num_sink=num_sink,
+                    mask_shift=mask_shift)
 
 
 def wrapped_flash_attn_fwd_varlen(
     q, k, v, softmax_scale, window_size, cu_seqlens_q, cu_seqlens_k,
-    max_seqlen_q=None, max_seqlen_k=None, causal=False, *, num_sink=0,
+    max_seqlen_q=None, max_seqlen_k=None, causal=False, *, num_sink=0, mask_shift=None,
 ):
     """Packed forward, ``ring_swa/ops/wrap_flash.py:203``.  ``max_seqlen_*`` are
     accepted for signature compatibility and unused (no host sync is needed)."""
     return attn_fwd(q, k, v, softmax_scale, window_size, causal, cu_seqlens_q, cu_seqlens_k,
-                    num_sink=num_sink)
+                    num_sink=num_sink, mask_shift=mask_shift)
 
 
 def wrapped_flash_attn_bwd(
-    q, k, v, o, softmax_lse, do, dq, dk, dv, softmax_scale, window_size, causal, *, num_sink=0
+    q, k, v, o, softmax_lse, do, dq, dk, dv, softmax_scale, window_size, causal, *, num_sink=0,
+    mask_shift=None,
 ):
     """Dense backward, ``ring_swa/ops/wrap_flash.py:276``; fills ``dq, dk, dv``."""
     attn_bwd(q, k, v, o, softmax_lse, do, dq, dk, dv, softmax_scale, window_size, causal,
-             num_sink=num_sink)
+             num_sink=num_sink, mask_shift=mask_shift)
 
 
 def wrapped_flash_attn_bwd_varlen(
     q, k, v, o, softmax_lse, do, dq, dk, dv, softmax_scale, window_size,
     cu_seqlens_q, cu_seqlens_k, max_seqlen_q=None, max_seqlen_k=None, causal=False, *,
-    num_sink=0,
+    num_sink=0, mask_shift=None,
 ):
     """Packed backward, ``ring_swa/ops/wrap_flash.py:330``; fills ``dq, dk, dv``."""
     attn_bwd(q, k, v, o, softmax_lse, do, dq, dk, dv, softmax_scale, window_size, causal,
-             cu_seqlens_q, cu_seqlens_k, num_sink=num_sink)
+             cu_seqlens_q, cu_seqlens_k, num_sink=num_sink, mask_shift=mask_shift)

@@ -57,6 +57,88 @@ def _incoming(rank: int, seq_len: int, window_size: int, cp_size: int, cu_host):
     return out
 
 
+def band_forward(q, kv, window_size, cp_group, cp_size, rank, softmax_scale, kernels, cu_host):
+    """Forward of the band blocks of one rank on ``[batch, seq, heads, dim]`` chunks (batch 1
+    around a packed chunk): returns the accumulators of
+    ``ring_swa/sliding_window/nonvarlen.py:53-59`` -- fp32 output, fp64 LSE -- before their
+    final cast, the device ``cu_seqlens`` of the own-chunk block (packed), the block plan and
+    the received key ranges by hop."""
+    b, s, hq, d = q.shape
+    local_cu, steps = _steps_of(rank, s, window_size, cp_size, cu_host)
+    cu_dev = None
+    if cu_host is not None:
+        cu_dev = torch.tensor(local_cu, dtype=torch.int32, device=q.device)
+    gmap = get_group_local_to_global_rank_map(cp_group)
+
+    # what this rank reads of earlier chunks / what later ranks read of this one
+    got = {}
+    recvs = []
+    for (i, _, ks, _, _) in steps:
+        if i > 0:
+            got[i] = kv.new_empty((2, b, ks.stop - ks.start, kv.shape[3], d))
+            recvs.append((got[i], gmap[rank - i]))
+    sends = [(kv[:, :, ks].contiguous(), gmap[other])
+             for (_, other, ks) in _incoming(rank, s, window_size, cp_size, cu_host)]
+    reqs = exchange(sends, recvs, cp_group)
+
+    out = torch.zeros_like(q, dtype=torch.float32)
+    lse = torch.full((b, hq, s), float("-inf"), dtype=torch.float64, device=q.device)
+    (_, _, _, window0, causal0) = steps[0]
+    if cu_host is not None:
+        flash_attn_varlen_fwd_func(q, kv, softmax_scale, window0, cu_dev, cu_dev, None, None,
+                                   causal0, out, lse, kernels=kernels)
+    else:
+        flash_attn_fwd_func(q, kv, softmax_scale, window0, causal0, out, lse, kernels=kernels)
+    for req in reqs:
+        req.wait()
+    for (i, qs, _, window, causal) in steps[1:]:
+        flash_attn_fwd_func(q[:, qs], got[i], softmax_scale, window, causal, out[:, qs],
+                            lse[:, :, qs], kernels=kernels)
+    return out, lse, cu_dev, steps, got
+
+
+def band_backward(q, kv, out, lse, do, got_list, window_size, cp_group, cp_size, rank,
+                  softmax_scale, kernels, cu_host, steps, cu_dev):
+    """Backward of the same blocks from the final ``(out, lse)``: fp32 ``dq`` and ``dkv`` of this
+    rank's chunk, the contributions of later ranks included."""
+    s = q.shape[1]
+    gmap = get_group_local_to_global_rank_map(cp_group)
+    dq = torch.zeros_like(q, dtype=torch.float32)
+    dkv = torch.zeros_like(kv, dtype=torch.float32)
+
+    # blocks on received key ranges first: their dKV goes back to the owners while the
+    # own-chunk block runs
+    sends = []
+    for (i, qs, _, window, causal), kv_i in zip(steps[1:], got_list):
+        dq_i = torch.empty_like(q[:, qs])
+        dkv_i = torch.empty_like(kv_i)
+        flash_attn_bwd_func(q[:, qs], kv_i, out[:, qs], lse[:, :, qs], do[:, qs], dq_i, dkv_i,
+                            softmax_scale, window, causal, kernels=kernels)
+        dq[:, qs] += dq_i
+        sends.append((dkv_i, gmap[rank - i]))
+    incoming = _incoming(rank, s, window_size, cp_size, cu_host)
+    back = [kv.new_empty((2, kv.shape[1], ks.stop - ks.start, kv.shape[3], kv.shape[4]))
+            for (_, _, ks) in incoming]
+    recvs = [(buf, gmap[other]) for buf, (_, other, _) in zip(back, incoming)]
+    reqs = exchange(sends, recvs, cp_group)
+
+    (_, _, _, window0, causal0) = steps[0]
+    dq_0, dkv_0 = torch.empty_like(q), torch.empty_like(kv)
+    if cu_host is not None:
+        flash_attn_varlen_bwd_func(q, kv, out, lse, do, dq_0, dkv_0, cu_dev, cu_dev, None, None,
+                                   softmax_scale, window0, causal0, kernels=kernels)
+    else:
+        flash_attn_bwd_func(q, kv, out, lse, do, dq_0, dkv_0, softmax_scale, window0, causal0,
+                            kernels=kernels)
+    dq += dq_0
+    dkv += dkv_0
+    for req in reqs:
+        req.wait()
+    for buf, (_, _, ks) in zip(back, incoming):  # hop order: a fixed order of the fp32 sums
+        dkv[:, :, ks] += buf
+    return dq, dkv
+
+
 class RingSlidingWindowFunc(torch.autograd.Function):
     """Dense ``[batch, seq, heads, dim]`` chunks, or packed ``[tokens, heads, dim]`` chunks
     when ``cu_host`` (the cumulative lengths of the WHOLE pack, a host list) is given."""
@@ -67,44 +149,13 @@ class RingSlidingWindowFunc(torch.autograd.Function):
         packed = cu_host is not None
         if packed:
             q, k, v = q.unsqueeze(0), k.unsqueeze(0), v.unsqueeze(0)
-        b, s, hq, d = q.shape
         if softmax_scale is None:
-            softmax_scale = d ** (-0.5)
-        local_cu, steps = _steps_of(rank, s, window_size, cp_size, cu_host)
-        cu_dev = None
-        if packed:
-            cu_dev = torch.tensor(local_cu, dtype=torch.int32, device=q.device)
-        gmap = get_group_local_to_global_rank_map(cp_group)
+            softmax_scale = q.shape[-1] ** (-0.5)
         kv = torch.stack([k, v], dim=0)
-
-        # what this rank reads of earlier chunks / what later ranks read of this one
-        got = {}
-        recvs = []
-        for (i, _, ks, _, _) in steps:
-            if i > 0:
-                got[i] = kv.new_empty((2, b, ks.stop - ks.start, kv.shape[3], d))
-                recvs.append((got[i], gmap[rank - i]))
-        sends = [(kv[:, :, ks].contiguous(), gmap[other])
-                 for (_, other, ks) in _incoming(rank, s, window_size, cp_size, cu_host)]
-        reqs = exchange(sends, recvs, cp_group)
-
-        # accumulators of ring_swa/sliding_window/nonvarlen.py:53-59
-        out = torch.zeros_like(q, dtype=torch.float32)
-        lse = torch.full((b, hq, s), float("-inf"), dtype=torch.float64, device=q.device)
-        (_, _, _, window0, causal0) = steps[0]
-        if packed:
-            flash_attn_varlen_fwd_func(q, kv, softmax_scale, window0, cu_dev, cu_dev, None, None,
-                                       causal0, out, lse, kernels=kernels)
-        else:
-            flash_attn_fwd_func(q, kv, softmax_scale, window0, causal0, out, lse, kernels=kernels)
-        for req in reqs:
-            req.wait()
-        for (i, qs, _, window, causal) in steps[1:]:
-            flash_attn_fwd_func(q[:, qs], got[i], softmax_scale, window, causal, out[:, qs],
-                                lse[:, :, qs], kernels=kernels)
+        out, lse, cu_dev, steps, got = band_forward(q, kv, window_size, cp_group, cp_size, rank,
+                                                    softmax_scale, kernels, cu_host)
         out = out.to(q.dtype)
         lse = lse.to(torch.float32)
-
         ctx.save_for_backward(q, kv, out, lse, *(got[i] for (i, *_rest) in steps[1:]))
         ctx.cu_dev = cu_dev
         ctx.meta = (window_size, cp_group, cp_size, rank, softmax_scale, kernels, cu_host, steps)
@@ -119,43 +170,8 @@ class RingSlidingWindowFunc(torch.autograd.Function):
             do = do.unsqueeze(0)
         if do.stride(-1) != 1:
             do = do.contiguous()
-        s = q.shape[1]
-        gmap = get_group_local_to_global_rank_map(cp_group)
-        dq = torch.zeros_like(q, dtype=torch.float32)
-        dkv = torch.zeros_like(kv, dtype=torch.float32)
-
-        # blocks on received key ranges first: their dKV goes back to the owners while the
-        # own-chunk block runs
-        sends = []
-        for (i, qs, _, window, causal), kv_i in zip(steps[1:], got_list):
-            dq_i = torch.empty_like(q[:, qs])
-            dkv_i = torch.empty_like(kv_i)
-            flash_attn_bwd_func(q[:, qs], kv_i, out[:, qs], lse[:, :, qs], do[:, qs], dq_i, dkv_i,
-                                softmax_scale, window, causal, kernels=kernels)
-            dq[:, qs] += dq_i
-            sends.append((dkv_i, gmap[rank - i]))
-        incoming = _incoming(rank, s, window_size, cp_size, cu_host)
-        back = [kv.new_empty((2, kv.shape[1], ks.stop - ks.start, kv.shape[3], kv.shape[4]))
-                for (_, _, ks) in incoming]
-        recvs = [(buf, gmap[other]) for buf, (_, other, _) in zip(back, incoming)]
-        reqs = exchange(sends, recvs, cp_group)
-
-        (_, _, _, window0, causal0) = steps[0]
-        dq_0, dkv_0 = torch.empty_like(q), torch.empty_like(kv)
-        if packed:
-            flash_attn_varlen_bwd_func(q, kv, out, lse, do, dq_0, dkv_0, ctx.cu_dev, ctx.cu_dev,
-                                       None, None, softmax_scale, window0, causal0,
-                                       kernels=kernels)
-        else:
-            flash_attn_bwd_func(q, kv, out, lse, do, dq_0, dkv_0, softmax_scale, window0, causal0,
-                                kernels=kernels)
-        dq += dq_0
-        dkv += dkv_0
-        for req in reqs:
-            req.wait()
-        for buf, (_, _, ks) in zip(back, incoming):  # hop order: a fixed order of the fp32 sums
-            dkv[:, :, ks] += buf
-
+        dq, dkv = band_backward(q, kv, out, lse, do, got_list, window_size, cp_group, cp_size,
+                                rank, softmax_scale, kernels, cu_host, steps, ctx.cu_dev)
         dq, dk, dv = dq.to(q.dtype), dkv[0].to(kv.dtype), dkv[1].to(kv.dtype)
         if packed:
             dq, dk, dv = dq.squeeze(0), dk.squeeze(0), dv.squeeze(0)

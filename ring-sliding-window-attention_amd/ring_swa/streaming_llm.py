@@ -33,16 +33,7 @@ import torch
 
 from .ops.band_attn import attn_bwd, attn_fwd
 from .ops.lse_merge import merge_attn_out
-from .sliding_window import BandAttnFunc, _check_dense, _check_packed
-
-
-def _reject_ring(cp_group):
-    if cp_group is not None:
-        raise NotImplementedError(
-            "streaming-LLM attention over a context-parallel group (sink broadcast, sink-gradient "
-            "reduction) is not part of this build; sliding-window attention is "
-            "(ring_swa.ring_sliding_window_attn[_varlen] with cp_group)"
-        )
+from .sliding_window import BandAttnFunc, _check_dense, _check_packed, _ring_ranks
 
 
 class SinkWindowSplitFunc(torch.autograd.Function):
@@ -145,10 +136,19 @@ def ring_streaming_llm_attn(
     num_sink_tokens: int = 1,
     impl: str = "fused",
 ) -> torch.Tensor:
-    """Sink + sliding-window attention on ``[batch, seq, heads, dim]`` tensors."""
-    _reject_ring(cp_group)
+    """Sink + sliding-window attention on ``[batch, seq, heads, dim]`` tensors.  With a
+    ``cp_group`` the tensors are this rank's chunk of the sequence (``ring_slm.py``; ``impl``
+    plays no role there)."""
     _check_dense(q, k, v)
     assert num_sink_tokens >= 0
+    _impl(impl)
+    if cp_group is not None:
+        from .ring_slm import ring_slm_attn
+
+        cp_size, cp_local_rank = _ring_ranks(cp_group, cp_size, cp_local_rank,
+                                             cp_prev_global_rank, cp_next_global_rank)
+        return ring_slm_attn(q, k, v, window_size, cp_group, cp_size, cp_local_rank,
+                             softmax_scale, num_sink_tokens=num_sink_tokens)
     if _impl(impl) or num_sink_tokens == 0:
         return BandAttnFunc.apply(q, k, v, int(window_size), softmax_scale, None,
                                   int(num_sink_tokens))
@@ -172,10 +172,19 @@ def ring_streaming_llm_attn_varlen(
     num_sink_tokens: int = 1,
     impl: str = "fused",
 ) -> torch.Tensor:
-    """Packed variant: ``[tokens, heads, dim]`` tensors, ``cu_seqlens`` int32 ``[B+1]``."""
-    _reject_ring(cp_group)
-    _check_packed(q, k, v, cu_seqlens, cp_size)
+    """Packed variant: ``[tokens, heads, dim]`` tensors, ``cu_seqlens`` int32 ``[B+1]`` (with a
+    ``cp_group``: of the whole pack, the tensors being this rank's chunk of it)."""
     assert num_sink_tokens >= 0
+    _impl(impl)
+    if cp_group is not None:
+        from .ring_slm import ring_slm_attn
+
+        _check_packed(q, k, v, cu_seqlens, 1)
+        cp_size, cp_local_rank = _ring_ranks(cp_group, cp_size, cp_local_rank,
+                                             cp_prev_global_rank, cp_next_global_rank)
+        return ring_slm_attn(q, k, v, window_size, cp_group, cp_size, cp_local_rank,
+                             softmax_scale, cu_seqlens, num_sink_tokens=num_sink_tokens)
+    _check_packed(q, k, v, cu_seqlens, cp_size)
     cu = cu_seqlens.contiguous()
     if _impl(impl) or num_sink_tokens == 0:
         return BandAttnFunc.apply(q, k, v, int(window_size), softmax_scale, cu,

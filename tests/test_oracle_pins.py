@@ -359,3 +359,20 @@ def test_global_mask_with_sinks_equals_the_per_sequence_rule():
                 for t in range(total):
                     rule = sid[p] == sid[t] and t <= p and (p - t <= w or t - cu[sid[t]] < n)
                     assert bool(got[p, t]) == bool(rule)
+
+
+def test_explicit_shift_of_the_window_rule_by_brute_force():
+    """``shift`` moves the diagonal: key j visible from row i iff j <= i + shift + right and
+    j >= i + shift - left (negative bound: none); the default is ``sk - sq``."""
+    for sq, sk, window, shift in ((7, 3, (-1, 0), -4), (5, 9, (2, 1), 0), (6, 6, (1, -1), 3),
+                                  (4, 2, (-1, 0), -9), (8, 8, (3, 0), None)):
+        got = O.window_allowed(sq, sk, window, False, shift=shift)
+        sh = sk - sq if shift is None else shift
+        for i in range(sq):
+            for j in range(sk):
+                want = True
+                if window[1] >= 0:
+                    want &= j <= i + sh + window[1]
+                if window[0] >= 0:
+                    want &= j >= i + sh - window[0]
+                assert bool(got[i, j]) == want, (sq, sk, window, shift, i, j)

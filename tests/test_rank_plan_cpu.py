@@ -70,14 +70,10 @@ def test_benchmark_geometry():
     assert RS.ring_comm_times(10 ** 6, 8192, 8) == 7
 
 
-def test_public_api_rejects_slm_ring_and_cpu():
+def test_public_api_rejects_cpu_tensors_and_bad_arguments():
     import ring_swa
 
     q = torch.zeros(1, 8, 4, 128, dtype=torch.bfloat16)
-    # sliding-window attention takes a cp_group (tests/test_ring_gloo_cpu.py); the
-    # streaming-LLM ring is not part of this build
-    with pytest.raises(NotImplementedError, match="context-parallel group"):
-        ring_swa.ring_streaming_llm_attn(q, q, q, 4, object())
     with pytest.raises(RuntimeError, match="no CPU path"):
         ring_swa.ring_sliding_window_attn(q, q, q, 4)
     with pytest.raises(AssertionError):

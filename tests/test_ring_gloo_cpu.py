@@ -29,15 +29,16 @@ def _free_port():
 def oracle_kernels(dtype=torch.float64):
     """The five primitives of ``ops/accum.py`` on the oracle (CPU, fp64)."""
 
-    def fwd(q, k, v, scale, window, causal):
-        return O.window_attention(q, k, v, scale, window, causal, compute_dtype=dtype)
+    def fwd(q, k, v, scale, window, causal, mask_shift=None):
+        return O.window_attention(q, k, v, scale, window, causal, compute_dtype=dtype,
+                                  shift=mask_shift)
 
     def fwd_varlen(q, k, v, scale, window, cu_q, cu_k, max_q, max_k, causal):
         return O.window_attention_varlen(q, k, v, cu_q.tolist(), cu_k.tolist(), scale, window,
                                          causal, compute_dtype=dtype)
 
-    def bwd(q, k, v, o, lse, do, dq, dk, dv, scale, window, causal):
-        allowed = O.window_allowed(q.shape[1], k.shape[1], window, causal)
+    def bwd(q, k, v, o, lse, do, dq, dk, dv, scale, window, causal, mask_shift=None):
+        allowed = O.window_allowed(q.shape[1], k.shape[1], window, causal, shift=mask_shift)
         a, b, c = O.attention_bwd_from_stats(q, k, v, o, lse, do, allowed, scale, dtype)
         dq.copy_(a), dk.copy_(b), dv.copy_(c)
 
@@ -81,18 +82,26 @@ def _worker(rank, world, port, cases, results):
             got = get_group_local_to_global_rank_map(sub)
             assert got == dict(enumerate(sorted(members))) or got == dict(enumerate(members)), got
             assert got[dist.get_rank(sub)] == rank
+    from ring_swa.ring_slm import ring_slm_attn
+
     K = oracle_kernels()
     out = {}
-    for name, (q, k, v, do, w, cu) in cases.items():
+    for name, (q, k, v, do, w, cu, *sinks) in cases.items():
         s = q.shape[-3] // world
         sl = slice(rank * s, (rank + 1) * s)
+        if sinks:
+            run = lambda a, b, c, cu_: ring_slm_attn(a, b, c, w, group, world, rank, None, cu_,  # noqa: E731
+                                                     num_sink_tokens=sinks[0], kernels=K)
+        else:
+            run = lambda a, b, c, cu_: ring_attn(a, b, c, w, group, world, rank, None, cu_,  # noqa: E731
+                                                 kernels=K)
         if cu is None:
             qr, kr, vr = (t[:, sl].clone().requires_grad_() for t in (q, k, v))
-            o = ring_attn(qr, kr, vr, w, group, world, rank, None, None, kernels=K)
+            o = run(qr, kr, vr, None)
             o.backward(do[:, sl])
         else:
             qr, kr, vr = (t[sl].clone().requires_grad_() for t in (q, k, v))
-            o = ring_attn(qr, kr, vr, w, group, world, rank, None, cu, kernels=K)
+            o = run(qr, kr, vr, cu)
             o.backward(do[sl])
         out[name] = (o.detach(), qr.grad, kr.grad, vr.grad)
     results[rank] = out
@@ -115,6 +124,19 @@ def _cases(world):
         q, do = (torch.randn(total, hq, d, generator=g, dtype=torch.float64) for _ in range(2))
         k, v = (torch.randn(total, hk, d, generator=g, dtype=torch.float64) for _ in range(2))
         cases[f"packed{n}_w{w}"] = (q, k, v, do, w, cu)
+    # streaming-LLM: sinks of one sequence spread over ranks, more sinks than a chunk holds,
+    # windows shorter and longer than a chunk; packs whose sequences start anywhere
+    for n_sink, w in ((1, 2), (3, s - 1), (2, s + 2), (s + 2, 1), (4, 3 * s), (0, 3)):
+        q, do = (torch.randn(2, total, hq, d, generator=g, dtype=torch.float64) for _ in range(2))
+        k, v = (torch.randn(2, total, hk, d, generator=g, dtype=torch.float64) for _ in range(2))
+        cases[f"slm_dense_n{n_sink}_w{w}"] = (q, k, v, do, w, None, n_sink)
+    for n, (n_sink, w, cuts) in enumerate(((1, 2, [1, 7]), (3, 1, [s - 1]), (2, s, [s, s + 1]),
+                                           (4, 2, []), (2, 3, list(range(2, total, 5))),
+                                           (5, 0, [s - 2, 2 * s - 1]))):
+        cu = [0] + [c for c in cuts if 0 < c < total] + [total]
+        q, do = (torch.randn(total, hq, d, generator=g, dtype=torch.float64) for _ in range(2))
+        k, v = (torch.randn(total, hk, d, generator=g, dtype=torch.float64) for _ in range(2))
+        cases[f"slm_packed{n}_n{n_sink}_w{w}"] = (q, k, v, do, w, cu, n_sink)
     return cases
 
 
@@ -126,12 +148,15 @@ def test_ring_over_gloo_equals_the_whole_sequence_oracle(world):
         results = manager.dict()
         mp.spawn(_worker, args=(world, port, cases, results), nprocs=world, join=True)
         results = dict(results)
-    for name, (q, k, v, do, w, cu) in cases.items():
+    for name, (q, k, v, do, w, cu, *sinks) in cases.items():
+        n_sink = sinks[0] if sinks else 0
         if cu is None:
-            fn = lambda q, k, v: O.sliding_window_attn(q, k, v, w, compute_dtype=torch.float64)  # noqa: E731
+            fn = lambda q, k, v: O.streaming_llm_attn(q, k, v, w, n_sink=n_sink,  # noqa: E731
+                                                      compute_dtype=torch.float64)
             cat = 1
         else:
-            fn = lambda q, k, v: O.sliding_window_attn_varlen(q, k, v, w, cu, compute_dtype=torch.float64)  # noqa: E731
+            fn = lambda q, k, v: O.streaming_llm_attn_varlen(q, k, v, w, cu, n_sink=n_sink,  # noqa: E731
+                                                             compute_dtype=torch.float64)
             cat = 0
         ro, _, rq, rk, rv = O.attention_fwd_bwd(fn, q, k, v, do)
         for idx, ref in enumerate((ro, rq, rk, rv)):

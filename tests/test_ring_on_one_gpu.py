@@ -42,6 +42,11 @@ def _cases(world):
         cases[f"dense_w{w}"] = (total, w, None)
     cases["packed_w200"] = (total, 200, [0, 5, s - 3, s + 130, total])
     cases[f"packed_w{2 * s}"] = (total, 2 * s, [0, total - 37, total])
+    # streaming-LLM (fourth entry: sink tokens per sequence)
+    cases["slm_dense_n4_w100"] = (total, 100, None, 4)
+    cases[f"slm_dense_n1_w{s + 70}"] = (total, s + 70, None, 1)
+    cases["slm_packed_n4_w50"] = (total, 50, [0, 5, s - 3, s + 130, total], 4)
+    cases["slm_packed_n2_w300"] = (total, 300, [0, s - 1, total], 2)
     return cases
 
 
@@ -55,18 +60,22 @@ def _worker(rank, world, port, cases, results):
 
     group = dist.new_group(list(range(world)))
     out = {}
-    for n, (name, (total, w, cu)) in enumerate(cases.items()):
+    for n, (name, (total, w, cu, *sinks)) in enumerate(cases.items()):
         q, k, v, do = _inputs(total, cu is not None, n)
         s = total // world
         sl = slice(rank * s, (rank + 1) * s)
+        kw = {"num_sink_tokens": sinks[0]} if sinks else {}
         if cu is None:
+            fn = ring_swa.ring_streaming_llm_attn if sinks else ring_swa.ring_sliding_window_attn
             qr, kr, vr = (t[:, sl].cuda().requires_grad_() for t in (q, k, v))
-            o = ring_swa.ring_sliding_window_attn(qr, kr, vr, w, group)
+            o = fn(qr, kr, vr, w, group, **kw)
             o.backward(do[:, sl].cuda())
         else:
+            fn = (ring_swa.ring_streaming_llm_attn_varlen if sinks
+                  else ring_swa.ring_sliding_window_attn_varlen)
             qr, kr, vr = (t[sl].cuda().requires_grad_() for t in (q, k, v))
             cu_dev = torch.tensor(cu, dtype=torch.int32, device="cuda")
-            o = ring_swa.ring_sliding_window_attn_varlen(qr, kr, vr, w, cu_dev, group, world, rank)
+            o = fn(qr, kr, vr, w, cu_dev, group, world, rank, **kw)
             o.backward(do[sl].cuda())
         torch.cuda.synchronize()
         out[name] = tuple(t.detach().float().cpu() for t in (o, qr.grad, kr.grad, vr.grad))
@@ -85,15 +94,18 @@ def test_ring_ranks_on_one_gpu_equal_the_single_call(world):
         results = manager.dict()
         mp.spawn(_worker, args=(world, port, cases, results), nprocs=world, join=True)
         results = dict(results)
-    for n, (name, (total, w, cu)) in enumerate(cases.items()):
+    for n, (name, (total, w, cu, *sinks)) in enumerate(cases.items()):
         q, k, v, do = _inputs(total, cu is not None, n)
         qg, kg, vg = (t.cuda().requires_grad_() for t in (q, k, v))
+        kw = {"num_sink_tokens": sinks[0]} if sinks else {}
         if cu is None:
-            ref = ring_swa.ring_sliding_window_attn(qg, kg, vg, w)
+            fn = ring_swa.ring_streaming_llm_attn if sinks else ring_swa.ring_sliding_window_attn
+            ref = fn(qg, kg, vg, w, **kw)
             cat = 1
         else:
-            ref = ring_swa.ring_sliding_window_attn_varlen(
-                qg, kg, vg, w, torch.tensor(cu, dtype=torch.int32, device="cuda"))
+            fn = (ring_swa.ring_streaming_llm_attn_varlen if sinks
+                  else ring_swa.ring_sliding_window_attn_varlen)
+            ref = fn(qg, kg, vg, w, torch.tensor(cu, dtype=torch.int32, device="cuda"), **kw)
             cat = 0
         ref.backward(do.cuda())
         refs = [t.detach().float().cpu() for t in (ref, qg.grad, kg.grad, vg.grad)]
