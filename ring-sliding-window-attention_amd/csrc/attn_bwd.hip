@@ -7,9 +7,9 @@
 //          both fp32, into the caller's workspace
 //   DKDV : one block (4 waves, one per SIMD, up to 512 registers each) owns 256 keys of one
 //          (sequence, kv head) and walks the query tiles (32 rows) that can see them, for
-//          every q head of the GQA group; a wave owns 64 keys: their K fragments stay in
-//          registers, their V rows in LDS, dK^T / dV^T accumulate in accumulation registers
-//          for the whole walk and are written once
+//          every q head of the GQA group; a wave owns 64 keys: their K and V fragments stay
+//          in registers, dK^T / dV^T accumulate in accumulation registers for the whole
+//          walk and are written once
 //   DQ   : one block (8 waves x 32 query rows: 128 rows of two q heads of a GQA group, or
 //          256 rows of one head) walks the key tiles (64 keys) it can see, like the forward
 //          kernel; dQ^T stays in registers
@@ -21,7 +21,7 @@
 //
 // DKDV per (query tile, wave) (C layout: lane = key; two 32-key blocks per wave, so every
 // fragment read from LDS feeds two MFMAs):
-//   S = Q K^T, dP = dO V^T      A = Q / dO row fragments (LDS), B = K (registers) / V (LDS)
+//   S = Q K^T, dP = dO V^T      A = Q / dO row fragments (LDS), B = K / V (registers)
 //   P = exp2(S*c - lse2), dS = P * (dP - delta); the dP chains start from -delta instead of zero.
 //   (Folding c into 16-bit K fragments and starting the S chains from -lse2 would save the
 //   multiply-add per score -- 1-2 % -- but the rounding of K c shifts the exponent by up to
@@ -67,7 +67,6 @@ struct DkvCfg {
   static constexpr int CPR = D / 8;   // 16-byte chunks per row
   static constexpr int ROWB = D * 2;  // bytes per row
   static constexpr int Q_TILE = BM * ROWB;
-  static constexpr int V_TILE = BN * ROWB;
 };
 
 template <typename T, int D, bool SPLIT, bool FAR>
@@ -76,7 +75,6 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   using M = Mma<T>;
   using V8 = typename M::V8;
   constexpr int KB = C::KB, KS = C::KSTEPS, DB = C::DBLK;
-  __shared__ __attribute__((aligned(1024))) char v_s[C::V_TILE];
   __shared__ __attribute__((aligned(1024))) char q_s0[C::Q_TILE];
   __shared__ __attribute__((aligned(1024))) char q_s1[C::Q_TILE];
   __shared__ __attribute__((aligned(1024))) char do_s0[C::Q_TILE];
@@ -166,6 +164,20 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
     }
   }
 
+  // ... and so do its V fragments (B operand of dP = dO V^T, same layout)
+  V8 vf[KB][KS];
+#pragma unroll
+  for (int kb = 0; kb < KB; kb++) {
+    const int jc = jw0 + kb * 32 + l32;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      if (jc < len_k) {
+        vf[kb][ks] = *(const V8*)(v_ptr + (int64_t)jc * a.v_st[1] + ks * 16 + g * 8);
+      } else {
+        vf[kb][ks] = V8{0, 0, 0, 0, 0, 0, 0, 0};
+      }
+    }
+  }
   f32x16 dk_acc[KB][DB], dv_acc[KB][DB];
 #pragma unroll
   for (int kb = 0; kb < KB; kb++)
@@ -177,9 +189,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
         dv_acc[kb][d][i] = 0.f;
       }
   // ---- tile DMA (rows past the end of the sequence read as zero) ------------------
-  TileDma<D, C::BN, C::THREADS> v_dma;
   TileDma<D, C::BM, C::THREADS> q_dma, do_dma;
-  v_dma.init(a.v_st[1], tid);
   q_dma.init(a.q_st[1], tid);
   do_dma.init(a.do_st[1], tid);
   const T* q_base = (const T*)a.q + b * a.q_st[0] + s.q_row0 * a.q_st[1];
@@ -217,6 +227,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   // one at a time between the first MFMAs of a step; advance() then moves the cursor on.
   constexpr int NQD = TileDma<D, C::BM, C::THREADS>::N;
   constexpr int NPART = 1 + 2 * NQD;
+  const int st_voff = ((lane & 31) << 2) + (lane >> 5) * (stat_elems * 4);
   auto load_part = [&](int part, char* qd, char* dod, float* std_) __attribute__((always_inline)) {
     if (part == 0) {
       if (wave == 0) {  // lanes 0-31: lse2 of the 32 rows, lanes 32-63: their delta
@@ -226,10 +237,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
         // the per-lane offset is recomputed here (opaque to the optimiser): kept in a
         // register across the walk it could be spilled, and its reload would wait for
         // every tile load issued before it
-        int l = lane;
-        asm volatile("" : "+v"(l));
-        const int voff = ((l & 31) << 2) + (l >> 5) * (stat_elems * 4);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(st_rsrc, (lds_void_t*)std_, 4, voff, 0, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(st_rsrc, (lds_void_t*)std_, 4, st_voff, 0, 0, 0);
       }
     } else if (part <= NQD) {
       const TileSrc t = tile_src<C::BM, FAR>(nxt.q_head, nxt.i0, len_q, q_row_bytes, C::ROWB);
@@ -257,15 +265,12 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   };
 
   if (n_iter > 0) {
-    // (once per block: always based at the tile)
-    v_dma.load(tile_src<C::BN, true>(v_ptr, j0, len_k, (int)(a.v_st[1] * 2), C::ROWB), v_s);
 #pragma unroll
     for (int part = 0; part < NPART; part++) load_part(part, q_s0, do_s0, st_s0);
-    advance();
+    if (n_iter > 1) advance();
   }
   __syncthreads();
 
-  const char* v_lds = v_s + wave * (32 * KB) * C::ROWB;
 
   int cur_i0 = i_first + qt_start * C::BM;  // first row of the tile being computed
   // For which first rows i0 of a 32-row tile does any (query, key of this wave) pair survive
@@ -294,26 +299,25 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
     if (!needed && has_next) {
 #pragma unroll
       for (int part = 0; part < NPART; part++) load_part(part, qn, don, stn);
-      advance();
+      if (it + 2 < n_iter) advance();
     }
     if (needed) {
       const bool full = i0 >= full_lo && i0 <= full_hi;
-      const int rel_hi = (a.wr < 0) ? kInf : a.wr;
       // The four GEMMs of the (32 queries x 64 keys) sub-tile -- S = Q K^T, dP = dO V^T,
       // dV^T += dO^T P, dK^T += Q^T dS; KB KS MFMAs each, rows = queries, lane = key column
       // -- their LDS reads and the vector work are written out in issue order, one group
       // per MFMA, with scheduling fences between the groups.  Every fragment read from LDS
-      // feeds the MFMAs of both key blocks; K comes from registers; fragments are fetched
+      // feeds the MFMAs of both key blocks; K and V come from registers; fragments are fetched
       // AH fragment slots ahead; P = exp2(S c - lse2) is computed under the dP MFMAs and
       // dS = P (dP - delta) under the dV MFMAs; dP - delta comes out of the MFMAs, whose
       // chains start from -delta in the accumulator layout.
       constexpr int NG = KB * KS;   // MFMAs per GEMM (KS = 2 DB)
-      constexpr int NF = 4 * KS;    // fragment slots: Q, dO (+ V), dO^T, Q^T; KB MFMAs each
+      constexpr int NF = 4 * KS;    // fragment slots: Q, dO, dO^T, Q^T; KB MFMAs each
       constexpr int AH = 2;
       constexpr int GPC = NG / (4 * KB);  // MFMA groups per chunk of vector work
       static_assert(KS == 2 * DB && KB == 2, "GEMM shapes");
       auto fence = []() __attribute__((always_inline)) { __builtin_amdgcn_sched_barrier(0); };
-      V8 fa[NF], fv[KB][KS];
+      V8 fa[NF];
       auto fetch = [&](auto fc) __attribute__((always_inline)) {
         constexpr int f = decltype(fc)::value;
         if constexpr (f < KS) {
@@ -321,9 +325,6 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
         } else if constexpr (f < 2 * KS) {
           constexpr int ks = f - KS;
           fa[f] = *(const V8*)(doc + (a_row ^ (ks << 5)));
-#pragma unroll
-          for (int kb = 0; kb < KB; kb++)
-            fv[kb][ks] = *(const V8*)(v_lds + (a_row ^ (ks << 5)) + kb * 32 * C::ROWB);
         } else if constexpr (f < NF) {
           constexpr int j = (f - 2 * KS) % KS, ks2 = j / DB, d = j % DB;
           const char* src = f < 3 * KS ? doc : qc;
@@ -333,7 +334,9 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
         }
       };
       f32x16 sacc[KB], pacc[KB];
-      f32x16 dinit;  // -delta of the 32 rows in the accumulator layout: the dP chains start from it
+      // -delta of the 32 rows in the accumulator layout, from which the dP chains start, is read
+      // into the second key block's accumulator: the first block's chain takes it as a separate
+      // start operand, the second block's chain then accumulates in place
       f32x4 l4[4];   // -lse2 of the rows
       V8 pb[KB][2], dsb[KB][2];
       // vector work in 2 KB chunks of four rows: chunk order lets the packed operands of
@@ -352,20 +355,6 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
         for (int e = 0; e < 4; e++) {
           const int i = 4 * i4 + e;
           pk[kb][i] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][i], a.scale_log2, l4[i4][e]));
-        }
-        if (!full) {
-          // key position relative to the aligned diagonal of row i0: rel(r) = rel0 - r
-          const int jc = jw0 + kb * 32 + l32;
-          const int rel0 = jc - i0 - shift;
-          const int rel_lo = (a.wl < 0) ? -kInf : -a.wl;
-          const int rows_ok = (jc < len_k) ? len_q - i0 : 0;  // rows r < rows_ok are real
-#pragma unroll
-          for (int e = 0; e < 4; e++) {
-            const int r = 8 * i4 + 4 * g + e;
-            const int rel = rel0 - r;
-            const bool ok = (r < rows_ok) & (rel <= rel_hi) & (rel >= rel_lo);
-            pk[kb][4 * i4 + e] = ok ? pk[kb][4 * i4 + e] : 0.f;
-          }
         }
         if (i4 & 1) pb[kb][i4 >> 1] = M::pack(&pk[kb][8 * (i4 >> 1)]);
       };
@@ -387,25 +376,55 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
         constexpr int m = decltype(mc)::value;
         constexpr int f = m / KB, kb = m % KB;  // fragment slot and key block of this MFMA
         if constexpr (kb == 0) fetch(std::integral_constant<int, f + AH>{});
-        if (m < NPART && has_next) load_part(m, qn, don, stn);
+        // (after the last tile the cursor still names it: its rows are fetched once more, into
+        // the idle buffers, rather than branching around every load)
+        if constexpr (m < NPART) load_part(m, qn, don, stn);
         // row statistics: -delta early in S (the dP chains start from it), -lse2 at its end
         if constexpr (m >= 4 && m < 8) {
           const f32x4 t4 = *(const f32x4*)(delta_lds + 8 * (m - 4) + 4 * g);
 #pragma unroll
-          for (int e = 0; e < 4; e++) dinit[4 * (m - 4) + e] = t4[e];
+          for (int e = 0; e < 4; e++) pacc[KB - 1][4 * (m - 4) + e] = t4[e];
         }
         if constexpr (m >= NG - 4 && m < NG) l4[m - (NG - 4)] = *(const f32x4*)(lse_lds + 8 * (m - (NG - 4)) + 4 * g);
         if constexpr (m < NG) {
           if constexpr (f == 0) {
-            M::mfma32_vec0(fa[f], kf[kb][f], sacc[kb]);
+            if (full) {
+              M::mfma32_vec0(fa[f], kf[kb][f], sacc[kb]);
+            } else {
+              // The mask enters as the start value of the S chain: 0 for a visible pair, -inf
+              // otherwise (P = exp2(-inf) = 0, hence dS = 0).  Row r = c + 4 g of the tile, c
+              // fixed per register, is visible from key jc iff rmin <= r <= rmax with
+              //   rmin = t - rel_hi, rmax = min(t - rel_lo, rows_ok - 1), t = jc - i0 - shift:
+              // one unsigned comparison of r - rmin against the width of that interval.
+              constexpr int kBig = 1 << 29;  // |t| stays below it
+              const int rel_lo = (a.wl < 0) ? -kBig : -a.wl;
+              const int rel_up = (a.wr < 0) ? kBig : a.wr;
+              const int jc = jw0 + kb * 32 + l32;
+              const int t = jc - i0 - shift;
+              const int rows_ok = (jc < len_k) ? len_q - i0 : 0;  // rows r < rows_ok are real
+              const int rmin = t - rel_up;
+              const int rmax = min(t - rel_lo, rows_ok - 1);
+              const unsigned width = (unsigned)max(rmax - rmin + 1, 0);
+              const int base = 4 * g - rmin;
+#pragma unroll
+              for (int i = 0; i < 16; i++) {
+                const int c = 8 * (i >> 2) + (i & 3);
+                sacc[kb][i] = ((unsigned)(base + c) < width) ? 0.f : -__builtin_inff();
+              }
+              M::mfma32_vec(fa[f], kf[kb][f], sacc[kb]);
+            }
           } else {
             M::mfma32_vec(fa[f], kf[kb][f], sacc[kb]);
           }
         } else if constexpr (m < 2 * NG) {
           if constexpr (f == KS) {
-            M::mfma32_vec_init(fa[f], fv[kb][f - KS], dinit, pacc[kb]);
+            if constexpr (kb < KB - 1) {
+              M::mfma32_vec_init(fa[f], vf[kb][f - KS], pacc[KB - 1], pacc[kb]);
+            } else {
+              M::mfma32_vec(fa[f], vf[kb][f - KS], pacc[kb]);
+            }
           } else {
-            M::mfma32_vec(fa[f], fv[kb][f - KS], pacc[kb]);
+            M::mfma32_vec(fa[f], vf[kb][f - KS], pacc[kb]);
           }
           if constexpr ((m - NG + 1) % GPC == 0) p_chunk(std::integral_constant<int, (m - NG + 1) / GPC - 1>{});
         } else if constexpr (m < 3 * NG) {
@@ -419,7 +438,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
         }
         fence();
       });
-      if (has_next) advance();
+      if (it + 2 < n_iter) advance();
     }
     __syncthreads();
   };
