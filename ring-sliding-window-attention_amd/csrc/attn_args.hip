@@ -179,6 +179,10 @@ int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a, bool allow_
     };
     a.rev_q = keys_of(lq - 1) > keys_of(0);
     a.rev_k = rows_of(lk - 1) > rows_of(0);
+    // keys a query row sees on average (keys_of is piecewise linear: 17 samples)
+    int64_t sum = 0;
+    for (int t = 0; t <= 16; t++) sum += keys_of((lq - 1) * t / 16);
+    a.avg_keys = (int32_t)std::min<int64_t>(sum / 17, INT32_MAX);
   }
   a.scale = p->softmax_scale;
   a.scale_log2 = p->softmax_scale * kLog2e;

@@ -729,10 +729,16 @@ __global__ __launch_bounds__(256) void attn_bwd_sink_kernel(const AttnArgs a) {
 #ifndef RSWA_DQ_AH2
 #define RSWA_DQ_AH2 4
 #endif
+// dQ launches whose rows see at most this many keys on average use blocks of 4 waves, two per
+// compute unit (measured, 32 / 8 heads, head_dim 128: window 256 -22 %, window 1000 -8 %, the rank
+// step with its half-empty previous-chunk block -1.4 %; sequences of 16384 and more rows at
+// window 4096 +1 %; 32 = 32 heads, window 1000: -2 %)
+#ifndef RSWA_DQ_SMALL_AVG_KEYS
+#define RSWA_DQ_SMALL_AVG_KEYS 3200
+#endif
 template <int D>
 struct DqCfg {
   static constexpr int BN = 64;  // keys per step
-  static constexpr int THREADS = 512;
   static constexpr int KS = D / 32;   // k-steps of the 16x16x32 MFMAs over the head dim
   static constexpr int DB = D / 16;   // 16-row blocks of dQ^T
   static constexpr int KBLK = BN / 16;  // 16-key blocks per tile
@@ -751,9 +757,17 @@ struct DqCfg {
 // of neighbouring key blocks, packed, are the B operand of dQ^T += K^T dS^T over a 32-key slab
 // (k order: four keys of the first block, then four of the second); the A operand follows the
 // same order: two transposing reads, one per key block.
-template <typename T, int D, bool FAR>
-__global__ __launch_bounds__(512) void attn_bwd_dq_kernel(const AttnArgs a) {
+//
+// NW = 8: one block of 8 waves per compute unit (two waves per SIMD).  NW = 4: blocks of 4 waves,
+// two of them per compute unit -- the same two waves per SIMD, but from independent blocks, so
+// that one block's prologue (three dependent round trips to memory) and epilogue run under the
+// other's tiles; the price is that a K / V tile serves half as many rows.
+template <typename T, int D, bool FAR, int NW>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void attn_bwd_dq_kernel(const AttnArgs a) {
   using C = DqCfg<D>;
+  static_assert(NW == 8 || NW == 4, "waves per block");
+  constexpr int HSH = NW == 8 ? 2 : 1;  // waves per q head in pair mode: 1 << HSH
   using M = Mma<T>;
   using V8 = typename M::V8;
   constexpr int KS = C::KS, DB = C::DB, KBLK = C::KBLK;
@@ -774,17 +788,17 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(const AttnArgs a) {
   // row mode: the 8 waves take 256 consecutive rows of one q head
   const bool pair = (a.group & 1) == 0;
   const int units = pair ? a.group >> 1 : a.group;
-  const int bm = pair ? 128 : 256;
+  const int bm = pair ? 16 * NW : 32 * NW;
   const int hu = wid % units;
   int rest = wid / units;
   const int slot = a.rev_q ? a.n_tile - 1 - rest % a.n_tile : rest % a.n_tile;
   rest /= a.n_tile;
   const int hk = rest % a.heads_kv;
-  const int hq = hk * a.group + (pair ? 2 * hu + (wave >> 2) : hu);
+  const int hq = hk * a.group + (pair ? 2 * hu + (wave >> HSH) : hu);
   SeqInfo s;
   int qt;
   if (a.cu_q) {
-    if (!locate_packed(a, slot, pair ? 7 : 8, false, s, qt)) return;
+    if (!locate_packed(a, slot, (pair ? 4 : 5) + (NW == 8 ? 3 : 2), false, s, qt)) return;
   } else {
     s.batch_idx = rest / a.heads_kv;
     s.q_row0 = s.k_row0 = 0;
@@ -816,7 +830,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(const AttnArgs a) {
   const int n_tiles = n_sink_t + n_band;
   auto tile_of = [&](int it) { return it < n_sink_t ? it : t_lo + (it - n_sink_t); };
 
-  const int r0 = i0 + (pair ? wave & 3 : wave) * 32;
+  const int r0 = i0 + (pair ? wave & ((1 << HSH) - 1) : wave) * 32;
   const bool wave_valid = r0 < len_q;
   const bool wave_rows_full = r0 + 31 < len_q;
   const RowBounds wb_first = row_bounds(a, r0, len_q, len_k);
@@ -870,7 +884,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(const AttnArgs a) {
   const int rl = 4 * u + (r >> 2);
   const int t_row = rl * C::ROWB + ((((r & 3) >> 1) ^ swz16_f<C::CPR>(rl)) << 4) + (r & 1) * 8;
 
-  TileDma<D, C::BN, C::THREADS, true> k_dma, v_dma;
+  TileDma<D, C::BN, NW * 64, true> k_dma, v_dma;
   k_dma.init(a.k_st[1], tid);
   v_dma.init(a.v_st[1], tid);
   const int k_row_bytes = (int)(a.k_st[1] * 2), v_row_bytes = (int)(a.v_st[1] * 2);
@@ -1004,7 +1018,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(const AttnArgs a) {
   // ---- epilogue: dq = scale * acc, transposed through LDS for 16-byte stores ------
   // element i of dq_acc[d][qb] is dQ[query 16 qb + r][16 d + 4 u + i]
   char* stage = (wave & 3) == 0 ? k_s0 : (wave & 3) == 1 ? k_s1 : (wave & 3) == 2 ? v_s0 : v_s1;
-  for (int half = 0; half < 2; half++) {
+  for (int half = 0; half < NW / 4; half++) {
     if ((wave >> 2) == half) {
 #pragma unroll
       for (int d = 0; d < DB; d++)
@@ -1098,8 +1112,10 @@ __global__ __launch_bounds__(256) void attn_bwd_prep_kernel(const AttnArgs a) {
   template __global__ void attn_bwd_dkdv_kernel<T, D, true, false>(const AttnArgs);  \
   template __global__ void attn_bwd_dkdv_kernel<T, D, false, true>(const AttnArgs);  \
   template __global__ void attn_bwd_dkdv_kernel<T, D, true, true>(const AttnArgs);   \
-  template __global__ void attn_bwd_dq_kernel<T, D, false>(const AttnArgs);          \
-  template __global__ void attn_bwd_dq_kernel<T, D, true>(const AttnArgs);           \
+  template __global__ void attn_bwd_dq_kernel<T, D, false, 8>(const AttnArgs);       \
+  template __global__ void attn_bwd_dq_kernel<T, D, true, 8>(const AttnArgs);        \
+  template __global__ void attn_bwd_dq_kernel<T, D, false, 4>(const AttnArgs);       \
+  template __global__ void attn_bwd_dq_kernel<T, D, true, 4>(const AttnArgs);        \
   template __global__ void attn_bwd_sink_kernel<T, D>(const AttnArgs);                  \
   template __global__ void attn_bwd_prep_kernel<T, D>(const AttnArgs);
 RSWA_INSTANTIATE(__bf16, 128)
@@ -1150,9 +1166,9 @@ int launch_bwd(AttnArgs& a, hipStream_t stream, int phases) {
     }
   }
   if (phases & RSWA_BWD_DQ) {
-    using C = DqCfg<D>;
     const bool pair = (a.group & 1) == 0;
-    const int bm = pair ? 128 : 256;
+    const bool small = a.avg_keys <= RSWA_DQ_SMALL_AVG_KEYS;
+    const int bm = (pair ? 16 : 32) * (small ? 4 : 8);
     const int units_q = (pair ? a.group / 2 : a.group) * a.heads_kv;  // blocks per q tile
     if (a.cu_q) {
       a.n_tile = (int)(ceil_div(a.rows_q, bm) + a.batch);
@@ -1163,9 +1179,14 @@ int launch_bwd(AttnArgs& a, hipStream_t stream, int phases) {
     }
     if (a.n_work > 0) {
       clear_launch_error();
-      const dim3 grid(padded_grid(a.n_work)), block(C::THREADS);
-      if (a.far) hipLaunchKernelGGL((attn_bwd_dq_kernel<T, D, true>), grid, block, 0, stream, a);
-      else hipLaunchKernelGGL((attn_bwd_dq_kernel<T, D, false>), grid, block, 0, stream, a);
+      const dim3 grid(padded_grid(a.n_work)), block(small ? 256 : 512);
+      if (small) {
+        if (a.far) hipLaunchKernelGGL((attn_bwd_dq_kernel<T, D, true, 4>), grid, block, 0, stream, a);
+        else hipLaunchKernelGGL((attn_bwd_dq_kernel<T, D, false, 4>), grid, block, 0, stream, a);
+      } else {
+        if (a.far) hipLaunchKernelGGL((attn_bwd_dq_kernel<T, D, true, 8>), grid, block, 0, stream, a);
+        else hipLaunchKernelGGL((attn_bwd_dq_kernel<T, D, false, 8>), grid, block, 0, stream, a);
+      }
       int rc = check_launch("attn_bwd dq");
       if (rc != RSWA_OK) return rc;
     }

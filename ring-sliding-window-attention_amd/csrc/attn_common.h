@@ -63,6 +63,7 @@ struct AttnArgs {
   float* sink_part;
   int32_t* sink_count;
   int32_t sink_chunks;  // row chunks per (sequence, kv head)
+  int32_t avg_keys;  // keys a query row sees on average (host estimate; block shapes hang on it)
   int32_t far;  // a sequence of some streamed tensor spans 2 GiB or more: FAR kernels
   float scale, scale_log2;
 };
