@@ -36,9 +36,15 @@ struct FwdCfg {
   static_assert(TILE >= 32 * O_STRIDE, "one wave's epilogue staging fits one tile buffer");
 };
 
-template <typename T, int D, bool SKIP, bool FAR>
-__global__ __launch_bounds__(512) void attn_fwd_kernel(const AttnArgs a) {
+// NW = 8: the ping-pong block described above.  NW = 4: blocks of 4 waves in lock-step, two of
+// them per compute unit, for launches whose rows see few keys: a block's prologue and epilogue
+// then run under the other block's tiles, and a block's key range is narrower.
+template <typename T, int D, bool SKIP, bool FAR, int NW>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void attn_fwd_kernel(const AttnArgs a) {
   using C = FwdCfg<D>;
+  static_assert(NW == 8 || NW == 4, "waves per block");
+  constexpr int HSH = NW == 8 ? 2 : 1;  // waves per q head in pair mode: 1 << HSH
   using M = Mma<T>;
   using V8 = typename M::V8;
   __shared__ __attribute__((aligned(1024))) char k_s0[C::TILE];
@@ -61,17 +67,17 @@ __global__ __launch_bounds__(512) void attn_fwd_kernel(const AttnArgs a) {
   // row mode: the 8 waves take 256 consecutive rows of one q head
   const bool pair = (a.group & 1) == 0;
   const int units = pair ? a.group >> 1 : a.group;  // blocks per (kv head, q tile)
-  const int bm = pair ? 128 : 256;                  // query rows per block
+  const int bm = pair ? 16 * NW : 32 * NW;          // query rows per block
   const int hu = wid % units;
   int rest = wid / units;
   const int slot = a.rev_q ? a.n_tile - 1 - rest % a.n_tile : rest % a.n_tile;
   rest /= a.n_tile;
   const int hk = rest % a.heads_kv;
-  const int hq = hk * a.group + (pair ? 2 * hu + (wave >> 2) : hu);
+  const int hq = hk * a.group + (pair ? 2 * hu + (wave >> HSH) : hu);
   SeqInfo s;
   int qt;
   if (a.cu_q) {
-    if (!locate_packed(a, slot, pair ? 7 : 8, false, s, qt)) return;
+    if (!locate_packed(a, slot, (pair ? 4 : 5) + (NW == 8 ? 3 : 2), false, s, qt)) return;
   } else {
     s.batch_idx = rest / a.heads_kv;
     s.q_row0 = s.k_row0 = 0;
@@ -103,7 +109,7 @@ __global__ __launch_bounds__(512) void attn_fwd_kernel(const AttnArgs a) {
   auto tile_of = [&](int it) { return it < n_sink_t ? it : t_lo + (it - n_sink_t); };
 
   // ---- this wave's rows ----------------------------------------------------
-  const int r0 = i0 + (pair ? wave & 3 : wave) * 32;
+  const int r0 = i0 + (pair ? wave & ((1 << HSH) - 1) : wave) * 32;
   const int iq = r0 + l32;
   const RowBounds rb = row_bounds(a, iq, len_q, len_k);
   const bool wave_rows_full = r0 + 31 < len_q;
@@ -141,7 +147,7 @@ __global__ __launch_bounds__(512) void attn_fwd_kernel(const AttnArgs a) {
   const int t_row1 = (rl + 8) * C::ROWB + ((lp ^ swz_f<C::CPR>(rl + 8)) << 4) + (i16 & 1) * 8;
 
   // ---- tile DMA: rows past len_k read as zero ---------------------------------
-  TileDma<D, C::BN, C::THREADS> k_dma, v_dma;
+  TileDma<D, C::BN, NW * 64> k_dma, v_dma;
   k_dma.init(a.k_st[1], tid);
   v_dma.init(a.v_st[1], tid);
   const int k_row_bytes = (int)(a.k_st[1] * 2), v_row_bytes = (int)(a.v_st[1] * 2);
@@ -256,7 +262,7 @@ __global__ __launch_bounds__(512) void attn_fwd_kernel(const AttnArgs a) {
   // Tile loads: the wave group that is in the phase slot after both groups have finished
   // reading K(t), V(t-1) issues K(t+2) and V(t+1) into those buffers and waits for them
   // before the barrier that precedes their first use, one full slot later.
-  const bool late = __builtin_amdgcn_readfirstlane(wave >> 2) != 0;
+  const bool late = NW == 8 && __builtin_amdgcn_readfirstlane(wave >> 2) != 0;
   f32x16 s_cur[2];
   auto prefetch = [&](int it, char* kfree, char* vn) __attribute__((always_inline)) {
     if (it + 2 < n_tiles) load_k(it + 2, kfree);
@@ -356,7 +362,7 @@ __global__ __launch_bounds__(512) void attn_fwd_kernel(const AttnArgs a) {
       lse_new = both_empty ? ninf : fmaxf(la, lb) + log1pf(__expf(-fabsf(diff)));
     }
     if (g == 0 && iq < len_q) lse_ptr[(int64_t)iq * a.lse_st[2]] = lse_new;
-    for (int half = 0; half < 2; half++) {
+    for (int half = 0; half < NW / 4; half++) {
       if ((wave >> 2) == half) {
 #pragma unroll
         for (int d = 0; d < C::DBLK; d++)
@@ -404,22 +410,31 @@ __global__ __launch_bounds__(512) void attn_fwd_kernel(const AttnArgs a) {
 
 // Explicit instantiations: with implicit instantiation alone this hipcc emits the host
 // launch stubs of only some of the four variants.
-#define RSWA_INSTANTIATE(T, D)                                               \
-  template __global__ void attn_fwd_kernel<T, D, false, false>(const AttnArgs); \
-  template __global__ void attn_fwd_kernel<T, D, true, false>(const AttnArgs);  \
-  template __global__ void attn_fwd_kernel<T, D, false, true>(const AttnArgs);  \
-  template __global__ void attn_fwd_kernel<T, D, true, true>(const AttnArgs);
+#define RSWA_INSTANTIATE(T, D)                                                   \
+  template __global__ void attn_fwd_kernel<T, D, false, false, 8>(const AttnArgs); \
+  template __global__ void attn_fwd_kernel<T, D, true, false, 8>(const AttnArgs);  \
+  template __global__ void attn_fwd_kernel<T, D, false, true, 8>(const AttnArgs);  \
+  template __global__ void attn_fwd_kernel<T, D, true, true, 8>(const AttnArgs);   \
+  template __global__ void attn_fwd_kernel<T, D, false, false, 4>(const AttnArgs); \
+  template __global__ void attn_fwd_kernel<T, D, true, false, 4>(const AttnArgs);  \
+  template __global__ void attn_fwd_kernel<T, D, false, true, 4>(const AttnArgs);  \
+  template __global__ void attn_fwd_kernel<T, D, true, true, 4>(const AttnArgs);
 RSWA_INSTANTIATE(__bf16, 128)
 RSWA_INSTANTIATE(__bf16, 64)
 RSWA_INSTANTIATE(_Float16, 128)
 RSWA_INSTANTIATE(_Float16, 64)
 #undef RSWA_INSTANTIATE
 
-template <typename T, int D>
-int launch_fwd(AttnArgs& a, hipStream_t stream) {
-  using C = FwdCfg<D>;
+// Launches whose rows see at most this many keys on average use the 4-wave blocks (measured,
+// 32 / 8 heads: head_dim 64 at window 1000 -22 %, head_dim 128 at window 1000 -4 %, the packed
+// rank slice at window 2048 +2 points; at window 4096 the two forms are equal)
+#ifndef RSWA_FWD_SMALL_AVG_KEYS
+#define RSWA_FWD_SMALL_AVG_KEYS 3200
+#endif
+template <typename T, int D, int NW>
+int launch_fwd_nw(AttnArgs& a, hipStream_t stream) {
   const bool pair = (a.group & 1) == 0;
-  const int bm = pair ? 128 : 256;
+  const int bm = (pair ? 16 : 32) * NW;
   const int units = (pair ? a.group / 2 : a.group) * a.heads_kv;  // blocks per q tile
   if (a.cu_q) {
     a.n_tile = (int)(ceil_div(a.rows_q, bm) + a.batch);
@@ -434,15 +449,20 @@ int launch_fwd(AttnArgs& a, hipStream_t stream) {
   const int64_t span = (a.wl < 0 || a.wr < 0) ? (int64_t)1 << 40 : (int64_t)a.wl + a.wr + 1;
   const bool skip = (bm - 32) * 10 >= span + bm;
   clear_launch_error();
-  const dim3 grid(padded_grid(a.n_work)), block(C::THREADS);
+  const dim3 grid(padded_grid(a.n_work)), block(NW * 64);
   if (skip) {
-    if (a.far) hipLaunchKernelGGL((attn_fwd_kernel<T, D, true, true>), grid, block, 0, stream, a);
-    else hipLaunchKernelGGL((attn_fwd_kernel<T, D, true, false>), grid, block, 0, stream, a);
+    if (a.far) hipLaunchKernelGGL((attn_fwd_kernel<T, D, true, true, NW>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((attn_fwd_kernel<T, D, true, false, NW>), grid, block, 0, stream, a);
   } else {
-    if (a.far) hipLaunchKernelGGL((attn_fwd_kernel<T, D, false, true>), grid, block, 0, stream, a);
-    else hipLaunchKernelGGL((attn_fwd_kernel<T, D, false, false>), grid, block, 0, stream, a);
+    if (a.far) hipLaunchKernelGGL((attn_fwd_kernel<T, D, false, true, NW>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((attn_fwd_kernel<T, D, false, false, NW>), grid, block, 0, stream, a);
   }
   return check_launch("attn_fwd");
+}
+template <typename T, int D>
+int launch_fwd(AttnArgs& a, hipStream_t stream) {
+  return a.avg_keys <= RSWA_FWD_SMALL_AVG_KEYS ? launch_fwd_nw<T, D, 4>(a, stream)
+                                               : launch_fwd_nw<T, D, 8>(a, stream);
 }
 
 }  // namespace
