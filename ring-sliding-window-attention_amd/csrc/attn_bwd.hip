@@ -471,6 +471,46 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   // the result does not depend on timing -- and writes dK, dV.  Nobody waits for anybody.
   constexpr int GROUPS = 2 * KB * DB * 4;  // value groups per lane
   f32x4* part_base = (f32x4*)a.dkv_part + (int64_t)unit * a.nsplit * (GROUPS * C::THREADS);
+  if constexpr (!SPLIT) {
+    // Through LDS, one 32-key block of one matrix at a time: in the accumulator layout a lane
+    // holds 4 consecutive d of one key, so a direct store instruction would touch 32 rows with
+    // 16 bytes each (256 such instructions per block; at short walks -- 40 steps per block at
+    // window 1000 and one q head per kv head -- they took a tenth of the kernel).  Each wave
+    // stages its block in the tile buffer nobody reads any more (rows of 16-byte chunks, chunk
+    // c of row r at position c ^ (r % chunks-per-row)), and stores whole rows, 16 bytes a lane.
+    char* stage = wave == 0 ? q_s0 : wave == 1 ? q_s1 : wave == 2 ? do_s0 : do_s1;
+    static_assert(C::Q_TILE >= 32 * C::ROWB, "a 32-key block fits a tile buffer");
+    const int wr_row = l32_e * C::ROWB + g_e * 8;
+    const int wr_swz = l32_e & (C::CPR - 1);
+#pragma unroll
+    for (int mtx = 0; mtx < 2; mtx++)
+#pragma unroll
+      for (int kb = 0; kb < KB; kb++) {
+        const float sc = mtx == 0 ? a.scale : 1.f;
+#pragma unroll
+        for (int d = 0; d < DB; d++)
+#pragma unroll
+          for (int i4 = 0; i4 < 4; i4++) {
+            const f32x16& acc = mtx == 0 ? dk_acc[kb][d] : dv_acc[kb][d];
+            *(typename M::V4*)(stage + wr_row + (((d * 4 + i4) ^ wr_swz) << 4)) =
+                M::pack4(acc[4 * i4] * sc, acc[4 * i4 + 1] * sc, acc[4 * i4 + 2] * sc,
+                         acc[4 * i4 + 3] * sc);
+          }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wave's own writes have landed
+        T* dst = mtx == 0 ? dk_ptr : dv_ptr;
+        const int64_t dst_st = mtx == 0 ? a.dk_st[1] : a.dv_st[1];
+#pragma unroll
+        for (int n = 0; n < 32 * C::CPR / 64; n++) {
+          const int idx = n * 64 + lane_e;
+          const int row = idx / C::CPR, c = idx % C::CPR;
+          const V8 val = *(const V8*)(stage + row * C::ROWB + ((c ^ (row & (C::CPR - 1))) << 4));
+          const int jc = jw0 + kb * 32 + row;
+          if (jc < len_k) *(V8*)(dst + (int64_t)jc * dst_st + c * 8) = val;
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // read before the next block overwrites
+      }
+    return;
+  }
   {
     // one running pointer (opaque to the optimiser, or it would keep 64 addresses in registers)
     f32x4* mine = part_base + (int64_t)part * (GROUPS * C::THREADS) + (wave * 64 + lane_e);
@@ -484,16 +524,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
           for (int i4 = 0; i4 < 4; i4++) {
             const f32x16& acc = mtx == 0 ? dk_acc[kb][d] : dv_acc[kb][d];
             const f32x4 val = {acc[4 * i4], acc[4 * i4 + 1], acc[4 * i4 + 2], acc[4 * i4 + 3]};
-            if constexpr (!SPLIT) {
-              emit(mtx, kb, d, i4, val);
-            } else {
-              *mine = val;
-              mine += C::THREADS;
-              asm volatile("" : "+v"(mine));
-            }
+            *mine = val;
+            mine += C::THREADS;
+            asm volatile("" : "+v"(mine));
           }
   }
-  if constexpr (!SPLIT) return;
   // Release: every wave waits for its own stores, then one thread makes the block's partial
   // sums visible device-wide and counts the block in.  Acquire on the other side: the block
   // that finds itself last drops what its compute unit and L2 may hold of those lines.
