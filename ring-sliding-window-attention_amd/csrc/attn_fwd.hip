@@ -295,30 +295,40 @@ void attn_fwd_kernel(const AttnArgs a) {
     }
     if (!late) wait_dma();
     lds_barrier();
-    if (!late) prefetch(it, kfree, vn);
+    if (NW == 8 || !(need_cur && need_next)) {
+      if (!late) prefetch(it, kfree, vn);
+    }
     if (need_cur && need_next) {
       // matrix phase as ONE basic block, LDS reads scheduled four fragments ahead of their MFMA
+      if constexpr (NW == 4) {
+        // the tile loads ride between the MFMAs, one every fourth: issued in a row they hold the
+        // wave for about 50 cycles apiece before its first MFMA.  No branch may split the block,
+        // so past the last tile the last one is fetched again, into a buffer nobody reads
+        load_k(min(it + 2, n_tiles - 1), kfree);
+        load_v(min(it + 1, n_tiles - 1), vn);
+      }
       pv_acc(vc, pb);
       qk(kn, s_cur);
       __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
-#pragma unroll
-      for (int i = 0; i < 12; i++) {
+      static_for<32>([&](auto ic) __attribute__((always_inline)) {
+        constexpr int i = decltype(ic)::value;
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-      }
-#pragma unroll
-      for (int i = 0; i < 16; i++) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      }
-      __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+        if constexpr (i < 12) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        else if constexpr (i < 28) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        if constexpr (NW == 4 && i % 4 == 1) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      });
     } else if (need_cur) {
       pv_acc(vc, pb);
     } else if (need_next) {
       qk(kn, s_cur);
     }
-    if (late) wait_dma();
-    lds_barrier();
+    // (the second barrier of a tile exists for the ping-pong of the 8-wave block only: with all
+    // waves in the same phase, the buffers a tile's loads overwrite were last read before the
+    // tile's first barrier)
+    if constexpr (NW == 8) {
+      if (late) wait_dma();
+      lds_barrier();
+    }
   };
 
   if (n_tiles > 0) {
