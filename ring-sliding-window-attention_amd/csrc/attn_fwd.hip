@@ -3,8 +3,9 @@
 //
 // Replaces flash-attn's forward as wrapped at ring_swa/ops/wrap_flash.py:168-273.
 //
-// One block = 8 waves x 32 query rows sharing every K/V tile it loads: either 128 rows of
-// TWO q heads of one GQA group (group size even) or 256 rows of one q head.  Per 64-key
+// One block = 4 waves x 32 query rows sharing every K/V tile it loads: either 64 rows of
+// TWO q heads of one GQA group (group size even) or 128 rows of one q head; two blocks fit a
+// compute unit (two waves per SIMD, from independent blocks).  Per 64-key
 // tile a wave computes S^T = K Q^T (keys x queries) with v_mfma_f32_32x32x16, so each
 // lane owns ONE query column: the row max / sum of the online softmax are in-lane
 // reductions plus a single half-wave exchange, and P^T is already laid out as the B
@@ -15,9 +16,13 @@
 // directly in LDS, issued one (V) and two (K) tiles ahead.  The buffers are SEPARATE
 // static __shared__ arrays and the tile loop is unrolled by two, so that every access
 // names its buffer statically: only then can the compiler tell that an in-flight load
-// does not alias the LDS reads of the current tile, and not wait for it.  The two waves
-// of a SIMD run half a tile apart (ping-pong, see the tile loop): the softmax of one is
-// executed under the MFMAs of the other.
+// does not alias the LDS reads of the current tile, and not wait for it.  The waves of a
+// block run in lock-step, one barrier per tile; the softmax of one block runs under the MFMAs
+// of the compute unit's other block, and a block's prologue and epilogue under the other's
+// tiles.  (An 8-wave block whose two halves ran half a tile apart -- the softmax of one half
+// under the MFMAs of the other, two barriers per tile -- measured 5 % slower at window 4096
+// and 24 % slower at head_dim 64 and window 1000: half the tile loads per row, but one
+// block per compute unit and nothing to cover its prologue and epilogue.)
 #include "attn_common.h"
 
 namespace rswa {
@@ -26,7 +31,7 @@ namespace {
 template <int D>
 struct FwdCfg {
   static constexpr int BN = 64;
-  static constexpr int THREADS = 512;
+  static constexpr int THREADS = 256;
   static constexpr int KSTEPS = D / 16;
   static constexpr int DBLK = D / 32;
   static constexpr int CPR = D / 8;   // 16-byte chunks per row
@@ -36,15 +41,11 @@ struct FwdCfg {
   static_assert(TILE >= 32 * O_STRIDE, "one wave's epilogue staging fits one tile buffer");
 };
 
-// NW = 8: the ping-pong block described above.  NW = 4: blocks of 4 waves in lock-step, two of
-// them per compute unit, for launches whose rows see few keys: a block's prologue and epilogue
-// then run under the other block's tiles, and a block's key range is narrower.
-template <typename T, int D, bool SKIP, bool FAR, int NW>
-__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
+template <typename T, int D, bool SKIP, bool FAR>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void attn_fwd_kernel(const AttnArgs a) {
   using C = FwdCfg<D>;
-  static_assert(NW == 8 || NW == 4, "waves per block");
-  constexpr int HSH = NW == 8 ? 2 : 1;  // waves per q head in pair mode: 1 << HSH
+  constexpr int NW = C::THREADS / 64;
   using M = Mma<T>;
   using V8 = typename M::V8;
   __shared__ __attribute__((aligned(1024))) char k_s0[C::TILE];
@@ -63,8 +64,8 @@ void attn_fwd_kernel(const AttnArgs a) {
   const int u = lane >> 4;
 
   // ---- which (sequence, kv head, q tile, q head(s)) -------------------------
-  // pair mode: waves 0-3 and 4-7 take the same 128 rows of two neighbouring q heads;
-  // row mode: the 8 waves take 256 consecutive rows of one q head
+  // pair mode: waves 0-1 and 2-3 take the same 64 rows of two neighbouring q heads;
+  // row mode: the 4 waves take 128 consecutive rows of one q head
   const bool pair = (a.group & 1) == 0;
   const int units = pair ? a.group >> 1 : a.group;  // blocks per (kv head, q tile)
   const int bm = pair ? 16 * NW : 32 * NW;          // query rows per block
@@ -73,11 +74,11 @@ void attn_fwd_kernel(const AttnArgs a) {
   const int slot = a.rev_q ? a.n_tile - 1 - rest % a.n_tile : rest % a.n_tile;
   rest /= a.n_tile;
   const int hk = rest % a.heads_kv;
-  const int hq = hk * a.group + (pair ? 2 * hu + (wave >> HSH) : hu);
+  const int hq = hk * a.group + (pair ? 2 * hu + (wave >> 1) : hu);
   SeqInfo s;
   int qt;
   if (a.cu_q) {
-    if (!locate_packed(a, slot, (pair ? 4 : 5) + (NW == 8 ? 3 : 2), false, s, qt)) return;
+    if (!locate_packed(a, slot, pair ? 6 : 7, false, s, qt)) return;
   } else {
     s.batch_idx = rest / a.heads_kv;
     s.q_row0 = s.k_row0 = 0;
@@ -109,7 +110,7 @@ void attn_fwd_kernel(const AttnArgs a) {
   auto tile_of = [&](int it) { return it < n_sink_t ? it : t_lo + (it - n_sink_t); };
 
   // ---- this wave's rows ----------------------------------------------------
-  const int r0 = i0 + (pair ? wave & ((1 << HSH) - 1) : wave) * 32;
+  const int r0 = i0 + (pair ? wave & 1 : wave) * 32;
   const int iq = r0 + l32;
   const RowBounds rb = row_bounds(a, iq, len_q, len_k);
   const bool wave_rows_full = r0 + 31 < len_q;
@@ -147,7 +148,7 @@ void attn_fwd_kernel(const AttnArgs a) {
   const int t_row1 = (rl + 8) * C::ROWB + ((lp ^ swz_f<C::CPR>(rl + 8)) << 4) + (i16 & 1) * 8;
 
   // ---- tile DMA: rows past len_k read as zero ---------------------------------
-  TileDma<D, C::BN, NW * 64> k_dma, v_dma;
+  TileDma<D, C::BN, C::THREADS> k_dma, v_dma;
   k_dma.init(a.k_st[1], tid);
   v_dma.init(a.v_st[1], tid);
   const int k_row_bytes = (int)(a.k_st[1] * 2), v_row_bytes = (int)(a.v_st[1] * 2);
@@ -254,15 +255,11 @@ void attn_fwd_kernel(const AttnArgs a) {
     }
   };
 
-  // ---- ping-pong tile loop ------------------------------------------------------------
-  // A wave alternates a vector phase (mask + softmax of tile t, rescale of O) and a matrix
-  // phase (O += P(t) V(t), S(t+1) = K(t+1) Q^T), with a block barrier after each.  Waves 4-7
-  // run one phase behind waves 0-3, so on every SIMD one wave is in its matrix phase
-  // while the other is in its vector phase and both pipes stay busy.
-  // Tile loads: the wave group that is in the phase slot after both groups have finished
-  // reading K(t), V(t-1) issues K(t+2) and V(t+1) into those buffers and waits for them
-  // before the barrier that precedes their first use, one full slot later.
-  const bool late = NW == 8 && __builtin_amdgcn_readfirstlane(wave >> 2) != 0;
+  // ---- tile loop ------------------------------------------------------------------------
+  // Per tile: a vector section (mask + softmax of tile t, rescale of O), the block barrier,
+  // a matrix section (O += P(t) V(t), S(t+1) = K(t+1) Q^T).  The barrier publishes K(t+1) and
+  // V(t), loaded during the previous matrix section, and releases the buffers of K(t) and
+  // V(t-1), last read before it: the loads of K(t+2) and V(t+1) into them follow it.
   f32x16 s_cur[2];
   auto prefetch = [&](int it, char* kfree, char* vn) __attribute__((always_inline)) {
     if (it + 2 < n_tiles) load_k(it + 2, kfree);
@@ -270,8 +267,8 @@ void attn_fwd_kernel(const AttnArgs a) {
   };
   // A tile the block visits may hold no key that this wave's 32 rows can see (the block's
   // key range is as wide as the window plus all its rows): the wave then skips the tile's
-  // work and only keeps the barriers.  With a short window that is a sizeable share: at
-  // window 1000 and 256 rows per block a wave needs 17 of the block's 20 tiles.
+  // work and only keeps the barrier.  With a short window that is a sizeable share: at
+  // window 256 and 128 rows per block a wave needs 5 of the block's 7 tiles.
   // (SKIP is chosen by the host for short windows only: with a long window the test costs
   // more than the rare skipped tile saves.)
   auto wave_needs = [&](int it) __attribute__((always_inline)) -> bool {
@@ -286,27 +283,23 @@ void attn_fwd_kernel(const AttnArgs a) {
     // computed from stale LDS contents and never used
     const bool need_cur = SKIP ? wave_needs(it) : true;
     const bool need_next = SKIP ? wave_needs(it + 1) : true;
-    if (late) prefetch(it, kfree, vn);
     V8 pb[4];
     if (need_cur) {
       mask(it, s_cur);
       const float alpha = softmax(s_cur, pb);
       rescale(alpha);
     }
-    if (!late) wait_dma();
+    wait_dma();
     lds_barrier();
-    if (NW == 8 || !(need_cur && need_next)) {
-      if (!late) prefetch(it, kfree, vn);
-    }
+    if (!(need_cur && need_next)) prefetch(it, kfree, vn);
     if (need_cur && need_next) {
-      // matrix phase as ONE basic block, LDS reads scheduled four fragments ahead of their MFMA
-      if constexpr (NW == 4) {
-        // the tile loads ride between the MFMAs, one every fourth: issued in a row they hold the
-        // wave for about 50 cycles apiece before its first MFMA.  No branch may split the block,
-        // so past the last tile the last one is fetched again, into a buffer nobody reads
-        load_k(min(it + 2, n_tiles - 1), kfree);
-        load_v(min(it + 1, n_tiles - 1), vn);
-      }
+      // matrix section as ONE basic block, LDS reads scheduled four fragments ahead of their
+      // MFMA.  The tile loads ride between the MFMAs, one every fourth: issued in a row they
+      // hold the wave for about 50 cycles apiece before its first MFMA.  No branch may split
+      // the block, so past the last tile the last one is fetched again, into a buffer nobody
+      // reads.
+      load_k(min(it + 2, n_tiles - 1), kfree);
+      load_v(min(it + 1, n_tiles - 1), vn);
       pv_acc(vc, pb);
       qk(kn, s_cur);
       __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
@@ -315,19 +308,12 @@ void attn_fwd_kernel(const AttnArgs a) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         if constexpr (i < 12) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
         else if constexpr (i < 28) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        if constexpr (NW == 4 && i % 4 == 1) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        if constexpr (i % 4 == 1) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
       });
     } else if (need_cur) {
       pv_acc(vc, pb);
     } else if (need_next) {
       qk(kn, s_cur);
-    }
-    // (the second barrier of a tile exists for the ping-pong of the 8-wave block only: with all
-    // waves in the same phase, the buffers a tile's loads overwrite were last read before the
-    // tile's first barrier)
-    if constexpr (NW == 8) {
-      if (late) wait_dma();
-      lds_barrier();
     }
   };
 
@@ -337,22 +323,18 @@ void attn_fwd_kernel(const AttnArgs a) {
   }
   if (n_tiles > 1) load_k(1, k_s1);
   __syncthreads();
-  if (late) lds_barrier();
   if (wave_needs(0)) qk(k_s0, s_cur);
-  lds_barrier();
   for (int it = 0; it < n_tiles; it += 2) {
     iter(it, k_s1, k_s0, v_s0, v_s1);
     if (it + 1 < n_tiles) iter(it + 1, k_s0, k_s1, v_s1, v_s0);
   }
-  if (!late) lds_barrier();
   __syncthreads();
 
   // ---- epilogue --------------------------------------------------------------
   const float l_tot = halfwave_sum(l_run);
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-  // transpose O^T through LDS for coalesced 16-byte stores: waves 0-3 first (one tile
-  // buffer each), then waves 4-7
-  char* stage = (wave & 3) == 0 ? k_s0 : (wave & 3) == 1 ? k_s1 : (wave & 3) == 2 ? v_s0 : v_s1;
+  // transpose O^T through LDS for coalesced 16-byte stores, one tile buffer per wave
+  char* stage = wave == 0 ? k_s0 : wave == 1 ? k_s1 : wave == 2 ? v_s0 : v_s1;
   // out_accumulate: out / lse hold a running partial result; the block is merged into it with
   // the arithmetic of the merge kernel (merge_lse.hip), applied to the block's output after
   // its rounding to 16 bits -- the same bits as a forward into a temporary plus a merge.  The
@@ -372,48 +354,42 @@ void attn_fwd_kernel(const AttnArgs a) {
       lse_new = both_empty ? ninf : fmaxf(la, lb) + log1pf(__expf(-fabsf(diff)));
     }
     if (g == 0 && iq < len_q) lse_ptr[(int64_t)iq * a.lse_st[2]] = lse_new;
-    for (int half = 0; half < NW / 4; half++) {
-      if ((wave >> 2) == half) {
+    // (the staging buffer is the wave's own: its writes only have to land before its reads)
 #pragma unroll
-        for (int d = 0; d < C::DBLK; d++)
+    for (int d = 0; d < C::DBLK; d++)
 #pragma unroll
-          for (int i4 = 0; i4 < 4; i4++) {
-            const auto h4 = M::pack4(o_acc[d][4 * i4] * inv, o_acc[d][4 * i4 + 1] * inv,
-                                     o_acc[d][4 * i4 + 2] * inv, o_acc[d][4 * i4 + 3] * inv);
-            *(typename M::V4*)(stage + l32 * C::O_STRIDE + (d * 32 + 8 * i4 + 4 * g) * 2) = h4;
-          }
-        if (g == 0) {
-          wgt[2 * l32] = w_old;
-          wgt[2 * l32 + 1] = w_new;
-        }
+      for (int i4 = 0; i4 < 4; i4++) {
+        const auto h4 = M::pack4(o_acc[d][4 * i4] * inv, o_acc[d][4 * i4 + 1] * inv,
+                                 o_acc[d][4 * i4 + 2] * inv, o_acc[d][4 * i4 + 3] * inv);
+        *(typename M::V4*)(stage + l32 * C::O_STRIDE + (d * 32 + 8 * i4 + 4 * g) * 2) = h4;
       }
-      __syncthreads();
-      if ((wave >> 2) == half) {
+    if (g == 0) {
+      wgt[2 * l32] = w_old;
+      wgt[2 * l32 + 1] = w_new;
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
-        for (int n = 0; n < 32 * C::CPR / 64; n++) {
-          const int c = lane + n * 64;
-          const int row = c / C::CPR, col = (c % C::CPR) * 8;
-          if (r0 + row < len_q) {
-            V8 val = *(const V8*)(stage + row * C::O_STRIDE + col * 2);
-            T* dst = o_ptr + (int64_t)(r0 + row) * a.o_st[1] + col;
-            if (a.out_accumulate) {
-              const float wo = wgt[2 * row], wn = wgt[2 * row + 1];
-              const V8 old = *(const V8*)dst;
-              float y[8];
+    for (int n = 0; n < 32 * C::CPR / 64; n++) {
+      const int c = lane + n * 64;
+      const int row = c / C::CPR, col = (c % C::CPR) * 8;
+      if (r0 + row < len_q) {
+        V8 val = *(const V8*)(stage + row * C::O_STRIDE + col * 2);
+        T* dst = o_ptr + (int64_t)(r0 + row) * a.o_st[1] + col;
+        if (a.out_accumulate) {
+          const float wo = wgt[2 * row], wn = wgt[2 * row + 1];
+          const V8 old = *(const V8*)dst;
+          float y[8];
 #pragma unroll
-              for (int j = 0; j < 8; j++) {
-                // a zero weight must annihilate whatever the other side holds
-                const float t0 = (wo == 0.f) ? 0.f : (float)old[j] * wo;
-                const float t1 = (wn == 0.f) ? 0.f : (float)val[j] * wn;
-                y[j] = t0 + t1;
-              }
-              val = M::pack(y);
-            }
-            *(V8*)dst = val;
+          for (int j = 0; j < 8; j++) {
+            // a zero weight must annihilate whatever the other side holds
+            const float t0 = (wo == 0.f) ? 0.f : (float)old[j] * wo;
+            const float t1 = (wn == 0.f) ? 0.f : (float)val[j] * wn;
+            y[j] = t0 + t1;
           }
+          val = M::pack(y);
         }
+        *(V8*)dst = val;
       }
-      __syncthreads();
     }
   }
 }
@@ -421,30 +397,21 @@ void attn_fwd_kernel(const AttnArgs a) {
 // Explicit instantiations: with implicit instantiation alone this hipcc emits the host
 // launch stubs of only some of the four variants.
 #define RSWA_INSTANTIATE(T, D)                                                   \
-  template __global__ void attn_fwd_kernel<T, D, false, false, 8>(const AttnArgs); \
-  template __global__ void attn_fwd_kernel<T, D, true, false, 8>(const AttnArgs);  \
-  template __global__ void attn_fwd_kernel<T, D, false, true, 8>(const AttnArgs);  \
-  template __global__ void attn_fwd_kernel<T, D, true, true, 8>(const AttnArgs);   \
-  template __global__ void attn_fwd_kernel<T, D, false, false, 4>(const AttnArgs); \
-  template __global__ void attn_fwd_kernel<T, D, true, false, 4>(const AttnArgs);  \
-  template __global__ void attn_fwd_kernel<T, D, false, true, 4>(const AttnArgs);  \
-  template __global__ void attn_fwd_kernel<T, D, true, true, 4>(const AttnArgs);
+  template __global__ void attn_fwd_kernel<T, D, false, false>(const AttnArgs); \
+  template __global__ void attn_fwd_kernel<T, D, true, false>(const AttnArgs);  \
+  template __global__ void attn_fwd_kernel<T, D, false, true>(const AttnArgs);  \
+  template __global__ void attn_fwd_kernel<T, D, true, true>(const AttnArgs);
 RSWA_INSTANTIATE(__bf16, 128)
 RSWA_INSTANTIATE(__bf16, 64)
 RSWA_INSTANTIATE(_Float16, 128)
 RSWA_INSTANTIATE(_Float16, 64)
 #undef RSWA_INSTANTIATE
 
-// Launches whose rows see at most this many keys on average use the 4-wave blocks (measured,
-// 32 / 8 heads: head_dim 64 at window 1000 -22 %, head_dim 128 at window 1000 -4 %, the packed
-// rank slice at window 2048 +2 points; at window 4096 the two forms are equal)
-#ifndef RSWA_FWD_SMALL_AVG_KEYS
-#define RSWA_FWD_SMALL_AVG_KEYS 3200
-#endif
-template <typename T, int D, int NW>
-int launch_fwd_nw(AttnArgs& a, hipStream_t stream) {
+template <typename T, int D>
+int launch_fwd(AttnArgs& a, hipStream_t stream) {
+  using C = FwdCfg<D>;
   const bool pair = (a.group & 1) == 0;
-  const int bm = (pair ? 16 : 32) * NW;
+  const int bm = pair ? 64 : 128;
   const int units = (pair ? a.group / 2 : a.group) * a.heads_kv;  // blocks per q tile
   if (a.cu_q) {
     a.n_tile = (int)(ceil_div(a.rows_q, bm) + a.batch);
@@ -459,20 +426,15 @@ int launch_fwd_nw(AttnArgs& a, hipStream_t stream) {
   const int64_t span = (a.wl < 0 || a.wr < 0) ? (int64_t)1 << 40 : (int64_t)a.wl + a.wr + 1;
   const bool skip = (bm - 32) * 10 >= span + bm;
   clear_launch_error();
-  const dim3 grid(padded_grid(a.n_work)), block(NW * 64);
+  const dim3 grid(padded_grid(a.n_work)), block(C::THREADS);
   if (skip) {
-    if (a.far) hipLaunchKernelGGL((attn_fwd_kernel<T, D, true, true, NW>), grid, block, 0, stream, a);
-    else hipLaunchKernelGGL((attn_fwd_kernel<T, D, true, false, NW>), grid, block, 0, stream, a);
+    if (a.far) hipLaunchKernelGGL((attn_fwd_kernel<T, D, true, true>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((attn_fwd_kernel<T, D, true, false>), grid, block, 0, stream, a);
   } else {
-    if (a.far) hipLaunchKernelGGL((attn_fwd_kernel<T, D, false, true, NW>), grid, block, 0, stream, a);
-    else hipLaunchKernelGGL((attn_fwd_kernel<T, D, false, false, NW>), grid, block, 0, stream, a);
+    if (a.far) hipLaunchKernelGGL((attn_fwd_kernel<T, D, false, true>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((attn_fwd_kernel<T, D, false, false>), grid, block, 0, stream, a);
   }
   return check_launch("attn_fwd");
-}
-template <typename T, int D>
-int launch_fwd(AttnArgs& a, hipStream_t stream) {
-  return a.avg_keys <= RSWA_FWD_SMALL_AVG_KEYS ? launch_fwd_nw<T, D, 4>(a, stream)
-                                               : launch_fwd_nw<T, D, 8>(a, stream);
 }
 
 }  // namespace
