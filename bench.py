@@ -30,8 +30,8 @@ PEAK_HBM_GBPS = 8000.0     # MI355X HBM3E
 # from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --pmc-pass`, each counter
 # scaled by what it reads for the 1 GiB device copy of that pass (FETCH_SIZE x2.0, WRITE_SIZE
 # x1.0); the summary is profiles/c3_own_chunk_kernels_hbm_traffic_pmc.txt.
-DKDV_HBM_BYTES_PER_LAUNCH = 274.4e6
-MERGE_HBM_BYTES_PER_LAUNCH = 5679.1e6
+DKDV_HBM_BYTES_PER_LAUNCH = 274.7e6
+MERGE_HBM_BYTES_PER_LAUNCH = 5681.3e6
 
 
 def band_pairs(length: int, w: int) -> int:
