@@ -120,18 +120,18 @@ typedef struct rswa_attn_params {
   int32_t heads_kv;
   int32_t seqlen_q; /* dense: exact; packed: upper bound of per-sequence len  */
   int32_t seqlen_k;
-  int64_t total_q;  /* packed mode only                                       */
+  int64_t total_q;  /* packed mode only; sequences stay below 2^28 rows       */
   int64_t total_k;
   const int32_t* cu_seqlens_q; /* NULL => dense                               */
   const int32_t* cu_seqlens_k;
 
   float softmax_scale;
-  int32_t window_left;  /* < 0: unbounded */
-  int32_t window_right; /* < 0: unbounded */
+  int32_t window_left;  /* < 0 (or >= 2^28): unbounded */
+  int32_t window_right; /* < 0 (or >= 2^28): unbounded */
   int32_t causal;
   int32_t num_sink;
   int32_t shift_explicit; /* 0: shift = len_k - len_q (flash-attn alignment) */
-  int32_t shift;          /* used when shift_explicit != 0                   */
+  int32_t shift;          /* used when shift_explicit != 0; |shift| < 2^28   */
 
   const void* q;
   const void* k;

@@ -150,8 +150,16 @@ int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a, bool allow_
   a.group = p->heads_q / p->heads_kv;
   a.seqlen_q = p->seqlen_q;
   a.seqlen_k = p->seqlen_k;
-  a.wl = p->window_left < 0 ? -1 : p->window_left;
-  a.wr = p->causal ? 0 : (p->window_right < 0 ? -1 : p->window_right);
+  // The kernels' mask arithmetic (row + shift +- window, key - row - shift) runs in 32 bits:
+  // lengths and an explicit shift stay below 2^28, and a window that reaches that far is the
+  // unbounded one.
+  constexpr int64_t kMaskLim = 1ll << 28;
+  RSWA_REQUIRE((packed ? std::max(p->total_q, p->total_k) : (int64_t)std::max(p->seqlen_q, p->seqlen_k)) < kMaskLim,
+               RSWA_ERR_UNSUPPORTED, "attn: sequences of 2^28 rows or more");
+  RSWA_REQUIRE(!p->shift_explicit || (p->shift > -kMaskLim && p->shift < kMaskLim), RSWA_ERR_UNSUPPORTED,
+               "attn: explicit mask shift %lld out of range (|shift| < 2^28)", (long long)p->shift);
+  a.wl = (p->window_left < 0 || p->window_left >= kMaskLim) ? -1 : p->window_left;
+  a.wr = p->causal ? 0 : ((p->window_right < 0 || p->window_right >= kMaskLim) ? -1 : p->window_right);
   a.n_sink = p->num_sink;
   a.shift_explicit = p->shift_explicit != 0;
   a.shift_val = p->shift;

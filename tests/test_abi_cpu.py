@@ -146,3 +146,29 @@ def test_what_stays_refused_beyond_2_gib_says_why():
     p.workspace_bytes = 0
     assert L.rswa_attn_bwd(p, None) == -1
     assert b"workspace" in L.rswa_last_error()
+
+
+def test_mask_arithmetic_limits_are_refused_or_mapped():
+    """The kernels compute masks in 32 bits: an explicit shift of 2^28 or more and sequences
+    that long are refused with a message; a window that reaches that far is the unbounded one
+    (the argument checks run before anything touches a device)."""
+    _ensure_built()
+    from ring_swa import _lib
+
+    L = _lib.lib()
+    p = _fake_params(1024)
+    p.shift_explicit, p.shift = 1, 1 << 28
+    assert L.rswa_attn_fwd(p, None) == -2
+    assert b"shift" in L.rswa_last_error()
+    p.shift = -(1 << 28)
+    assert L.rswa_attn_fwd(p, None) == -2
+    p = _fake_params(1 << 28, heads_q=1, heads_kv=1)
+    assert L.rswa_attn_fwd(p, None) == -2
+    assert b"2^28" in L.rswa_last_error()
+    # a window of 2^30 keys is accepted (it is the unbounded window): the backward's checks go
+    # on to the workspace
+    p = _fake_params(1024)
+    p.window_left = 1 << 30
+    p.workspace_bytes = 0
+    assert L.rswa_attn_bwd(p, None) == -1
+    assert b"workspace" in L.rswa_last_error()
