@@ -270,7 +270,7 @@ def _backward_blocks(q, k, v, prev_kv, out, lse, do, plan, scale, local_cu):
 def _backward_two_blocks(q, k, v, prev_kv, out, lse, do, plan, scale, local_cu):
     """Own-chunk block + one previous-chunk block (window no longer than a chunk): dq is
     summed inside the dQ kernel instead of in separate passes.  The previous-chunk block
-    writes its dQ first (side stream, onto zeros); the own-chunk dQ kernel, ordered after
+    writes its dQ first (side stream); the own-chunk dQ kernel, ordered after
     it, adds to it: fp32 sum of the two 16-bit partials, rounded once -- bit for bit what
     the fp32 accumulator of ring_swa/sliding_window/nonvarlen.py:203, 318-321 yields for two
     blocks.
@@ -285,8 +285,18 @@ def _backward_two_blocks(q, k, v, prev_kv, out, lse, do, plan, scale, local_cu):
     dK/dV launch take every compute unit first and loses that packing."""
     PREP, DKDV, DQ = 1, 2, 4
     (_, _, _, window0, causal0), (i1, qs, ks, window1, causal1) = plan
-    dq, dk, dv = torch.zeros_like(q), torch.empty_like(k), torch.empty_like(v)
-    dprev = [torch.zeros_like(kv) for kv in prev_kv]
+    # Only what no kernel writes is zeroed: the rows of dq outside the previous-chunk block (the
+    # own-chunk dQ kernel adds to every row), the rows of that chunk's dK / dV outside the block.
+    n_q, n_kv = q.shape[1], prev_kv[i1 - 1].shape[2]
+    q0, q1, _ = qs.indices(n_q)
+    k0, k1, _ = ks.indices(n_kv)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    dq[:, :q0].zero_()
+    dq[:, q1:].zero_()
+    dprev = [torch.empty_like(kv) if j == i1 - 1 else torch.zeros_like(kv)
+             for j, kv in enumerate(prev_kv)]
+    dprev[i1 - 1][:, :, :k0].zero_()
+    dprev[i1 - 1][:, :, k1:].zero_()
     kk, vv, dkv = prev_kv[i1 - 1][0], prev_kv[i1 - 1][1], dprev[i1 - 1]
     if local_cu is not None:
         need = bwd_workspace_bytes(q[0], k[0], local_cu, local_cu)
@@ -308,7 +318,7 @@ def _backward_two_blocks(q, k, v, prev_kv, out, lse, do, plan, scale, local_cu):
     def prev(phases):
         attn_bwd(q[:, qs], kk[:, ks], vv[:, ks], out[:, qs], lse[:, :, qs], do[:, qs], dq[:, qs],
                  dkv[0][:, ks], dkv[1][:, ks], scale, window1, causal1, workspace=ws_prev,
-                 phases=phases, dq_accumulate=True)
+                 phases=phases, dq_accumulate=False)
 
     side = _fork(q.device)
     with torch.cuda.stream(side):
