@@ -408,7 +408,8 @@ __device__ __forceinline__ float halfwave_sum(float x) {
 // prologue, partial store and share of the final sum -- so launches that already give every
 // compute unit a block are left alone.
 constexpr int kDkvKeysPerBlock = 256;
-constexpr int kMaxTileRows = 256;  // most rows any kernel fetches as one tile (V in dK/dV)
+constexpr int kMaxTileRows = 256;  // bound on the rows fetched as one tile that the stride checks assume
+                                   // (today's largest tile has 64 rows: K / V in the forward and dQ kernels)
 constexpr int kComputeUnits = 256;  // MI355X
 #ifndef RSWA_DKDV_SPLIT_BELOW
 #define RSWA_DKDV_SPLIT_BELOW (kComputeUnits / 2 + 1)
