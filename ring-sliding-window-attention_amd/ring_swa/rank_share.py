@@ -285,18 +285,14 @@ def _backward_two_blocks(q, k, v, prev_kv, out, lse, do, plan, scale, local_cu):
     dK/dV launch take every compute unit first and loses that packing."""
     PREP, DKDV, DQ = 1, 2, 4
     (_, _, _, window0, causal0), (i1, qs, ks, window1, causal1) = plan
-    # Only what no kernel writes is zeroed: the rows of dq outside the previous-chunk block (the
-    # own-chunk dQ kernel adds to every row), the rows of that chunk's dK / dV outside the block.
-    n_q, n_kv = q.shape[1], prev_kv[i1 - 1].shape[2]
-    q0, q1, _ = qs.indices(n_q)
-    k0, k1, _ = ks.indices(n_kv)
+    # Of dq only the rows outside the previous-chunk block are zeroed (the own-chunk dQ kernel
+    # adds to every row; the previous-chunk kernel writes the block's).  The previous chunk's
+    # dK / dV are zeroed whole: one contiguous fill is faster than a strided one of half the size.
+    q0, q1, _ = qs.indices(q.shape[1])
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     dq[:, :q0].zero_()
     dq[:, q1:].zero_()
-    dprev = [torch.empty_like(kv) if j == i1 - 1 else torch.zeros_like(kv)
-             for j, kv in enumerate(prev_kv)]
-    dprev[i1 - 1][:, :, :k0].zero_()
-    dprev[i1 - 1][:, :, k1:].zero_()
+    dprev = [torch.zeros_like(kv) for kv in prev_kv]
     kk, vv, dkv = prev_kv[i1 - 1][0], prev_kv[i1 - 1][1], dprev[i1 - 1]
     if local_cu is not None:
         need = bwd_workspace_bytes(q[0], k[0], local_cu, local_cu)
