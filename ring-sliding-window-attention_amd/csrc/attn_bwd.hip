@@ -1099,6 +1099,13 @@ __global__ __launch_bounds__(256) void attn_bwd_prep_kernel(const AttnArgs a) {
   // arrival counters of the dK/dV kernel's split blocks start from zero
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < a.n_count; i += (int64_t)gridDim.x * 256)
     a.dkv_count[i] = 0;
+  // The delta array starts at the next 256-byte boundary after the lse2 array, and the tile
+  // kernels read up to a tile of rows past the last one as statistics: the elements in between
+  // get the neutral value (P exactly zero) rather than whatever the workspace held.
+  if (blockIdx.x == 0) {
+    const int64_t used = a.rows_q * a.heads_q;
+    if (used + threadIdx.x < a.delta - a.lse2) a.lse2[used + threadIdx.x] = -__builtin_inff();
+  }
   const int64_t unit = ((int64_t)blockIdx.x * 256 + threadIdx.x) / LPR;  // (row, head)
   const int c = (threadIdx.x % LPR) * 8;
   if (unit >= a.rows_q * a.heads_q) return;

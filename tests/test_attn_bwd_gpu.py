@@ -259,6 +259,34 @@ def test_bwd_dq_accumulate_is_one_fp32_add_of_the_two_16bit_values(hq, hk, s):
     assert torch.equal(dk2, dk) and torch.equal(dv2, dv)
 
 
+@pytest.mark.parametrize("sq,sk,hq,hk,d,window", [
+    (300, 1000, 4, 4, 64, (-1, -1)),   # 2*300*4 statistics: 32 elements short of 256 bytes
+    (301, 301, 3, 1, 128, (50, 0)),
+    (77, 500, 5, 5, 128, (20, 0)),
+])
+def test_bwd_does_not_depend_on_what_the_workspace_held(sq, sk, hq, hk, d, window):
+    """The statistics arrays in the workspace are padded to 256 bytes and the tile kernels read
+    a tile of rows past a sequence's last one: whatever the caller's workspace held before (NaN
+    here, +inf, zeros) the results are the same bits."""
+    from ring_swa.ops import attn_bwd, attn_fwd
+    from ring_swa.ops.band_attn import bwd_workspace_bytes
+
+    g = torch.Generator().manual_seed(11)
+    q, do = (torch.randn(2, sq, hq, d, generator=g).bfloat16().cuda() for _ in range(2))
+    k, v = (torch.randn(2, sk, hk, d, generator=g).bfloat16().cuda() for _ in range(2))
+    out, lse = attn_fwd(q, k, v, None, window, True)
+    results = []
+    for fill in (float("nan"), float("inf"), 0.0):
+        ws = torch.full((bwd_workspace_bytes(q, k) // 4,), fill, device="cuda").view(torch.uint8)
+        dq, dk, dv = (torch.full_like(t, float("nan")) for t in (q, k, v))
+        attn_bwd(q, k, v, out, lse, do, dq, dk, dv, None, window, True, workspace=ws)
+        results.append((dq, dk, dv))
+    for dq, dk, dv in results:
+        for name, x, y in zip(("dq", "dk", "dv"), (dq, dk, dv), results[-1]):
+            assert torch.isfinite(x.float()).all(), name
+            assert torch.equal(x, y), name
+
+
 def test_bwd_empty_queries_write_only_the_outputs_of_the_requested_phases():
     """No query rows: dK = dV = 0 and dQ is empty, but a call restricted to the dQ phase
     must leave dK / dV (another call's results) alone."""
