@@ -174,7 +174,19 @@ typedef struct rswa_attn_params {
    * the kernel's epilogue: same bits as the two calls, one launch and one pass over out less
    * (what ring_swa/ops/attn.py:23-37 does with a temporary and a merge kernel). */
   int32_t out_accumulate;
-  int32_t reserved_;
+  /* Dense mode only.  > 0: the keys of the block are two row ranges of different tensors -- a
+   * ring rank's tail of the previous chunk followed by its own chunk -- taken as they lie,
+   * without concatenating them: key rows [0, seg_rows) are rows 0 .. of k / v (gradients: dk /
+   * dv), key rows [seg_rows, seqlen_k) are rows 0 .. of k2 / v2 (dk2 / dv2), which have the
+   * strides of k / v (dk / dv).  One kernel pass then covers what the reference computes as
+   * two blocks and a merge (ring_swa/sliding_window/nonvarlen.py:95-150: the own-chunk block
+   * and the previous chunk's corner).  seg_rows must be a multiple of 256 below seqlen_k, and
+   * num_sink 0.  0: one range, k2 .. dv2 ignored. */
+  int32_t seg_rows;
+  const void* k2;
+  const void* v2;
+  void* dk2;
+  void* dv2;
 } rswa_attn_params;
 
 #define RSWA_ADDR_AUTO 0

@@ -116,6 +116,30 @@ int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a, bool allow_
   a.dq = p->dq;
   a.dk = p->dk;
   a.dv = p->dv;
+  a.k2 = a.v2 = nullptr;
+  a.dk2 = a.dv2 = nullptr;
+  a.seg = INT32_MAX;
+  if (p->seg_rows != 0) {
+    RSWA_REQUIRE(!packed, RSWA_ERR_UNSUPPORTED, "attn: two key ranges (seg_rows) in dense mode only");
+    RSWA_REQUIRE(p->num_sink == 0, RSWA_ERR_UNSUPPORTED, "attn: two key ranges (seg_rows) with sink keys");
+    RSWA_REQUIRE(p->seg_rows > 0 && p->seg_rows % kDkvKeysPerBlock == 0 && p->seg_rows < p->seqlen_k,
+                 RSWA_ERR_UNSUPPORTED,
+                 "attn: seg_rows %d must be a positive multiple of %d below seqlen_k %d", p->seg_rows,
+                 kDkvKeysPerBlock, p->seqlen_k);
+    RSWA_REQUIRE(p->k2 && p->v2, RSWA_ERR_INVALID, "attn: seg_rows given but k2 / v2 null");
+    RSWA_REQUIRE(((uintptr_t)p->k2) % 16 == 0 && ((uintptr_t)p->v2) % 16 == 0, RSWA_ERR_UNSUPPORTED,
+                 "attn: k2 / v2 rows must start 16-byte aligned");
+    if (backward) {
+      RSWA_REQUIRE(p->dk2 && p->dv2, RSWA_ERR_INVALID, "attn_bwd: seg_rows given but dk2 / dv2 null");
+      RSWA_REQUIRE(((uintptr_t)p->dk2) % 16 == 0 && ((uintptr_t)p->dv2) % 16 == 0,
+                   RSWA_ERR_UNSUPPORTED, "attn_bwd: dk2 / dv2 rows must start 16-byte aligned");
+    }
+    a.k2 = p->k2;
+    a.v2 = p->v2;
+    a.dk2 = p->dk2;
+    a.dv2 = p->dv2;
+    a.seg = p->seg_rows;
+  }
   a.delta = nullptr;
   a.lse2 = nullptr;
   a.dkv_part = nullptr;

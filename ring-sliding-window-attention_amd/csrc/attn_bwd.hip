@@ -120,10 +120,15 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   const int j_last = min(j0 + C::BN, len_k) - 1;
   const int shift = a.shift_explicit ? a.shift_val : len_k - len_q;
 
-  const T* k_ptr = (const T*)a.k + b * a.k_st[0] + s.k_row0 * a.k_st[1] + hk * a.k_st[2];
-  const T* v_ptr = (const T*)a.v + b * a.v_st[0] + s.k_row0 * a.v_st[1] + hk * a.v_st[2];
-  T* dk_ptr = (T*)a.dk + b * a.dk_st[0] + s.k_row0 * a.dk_st[1] + hk * a.dk_st[2];
-  T* dv_ptr = (T*)a.dv + b * a.dv_st[0] + s.k_row0 * a.dv_st[1] + hk * a.dv_st[2];
+  // Keys in two row ranges (dense mode; the boundary is a multiple of the block's keys): the
+  // block's keys all lie in one of them, and its pointers are set so that a key's index in the
+  // sequence selects its row.
+  const bool seg2 = j0 >= a.seg;
+  const int64_t seg_row0 = seg2 ? -(int64_t)a.seg : s.k_row0;
+  const T* k_ptr = (const T*)(seg2 ? a.k2 : a.k) + b * a.k_st[0] + seg_row0 * a.k_st[1] + hk * a.k_st[2];
+  const T* v_ptr = (const T*)(seg2 ? a.v2 : a.v) + b * a.v_st[0] + seg_row0 * a.v_st[1] + hk * a.v_st[2];
+  T* dk_ptr = (T*)(seg2 ? a.dk2 : a.dk) + b * a.dk_st[0] + seg_row0 * a.dk_st[1] + hk * a.dk_st[2];
+  T* dv_ptr = (T*)(seg2 ? a.dv2 : a.dv) + b * a.dv_st[0] + seg_row0 * a.dv_st[1] + hk * a.dv_st[2];
   const int64_t ws_row0 = a.cu_q ? s.q_row0 : (int64_t)b * a.seqlen_q;
 
   // ---- query tiles that can see this key tile -------------------------------
@@ -923,10 +928,15 @@ void attn_bwd_dq_kernel(const AttnArgs a) {
   k_dma.init(a.k_st[1], tid);
   v_dma.init(a.v_st[1], tid);
   const int k_row_bytes = (int)(a.k_st[1] * 2), v_row_bytes = (int)(a.v_st[1] * 2);
+  // (keys in two row ranges: the second range's tensors, at this batch entry and kv head)
+  const T* k2_ptr = a.k2 ? (const T*)a.k2 + b * a.k_st[0] + hk * a.k_st[2] : k_ptr;
+  const T* v2_ptr = a.v2 ? (const T*)a.v2 + b * a.v_st[0] + hk * a.v_st[2] : v_ptr;
   auto load_tile = [&](int it, char* kd, char* vd) __attribute__((always_inline)) {
     const int j = tile_of(it) * C::BN;
-    k_dma.load(tile_src<C::BN, FAR>(k_ptr, j, len_k, k_row_bytes, C::ROWB), kd);
-    v_dma.load(tile_src<C::BN, FAR>(v_ptr, j, len_k, v_row_bytes, C::ROWB), vd);
+    const KeySeg<T> gk = key_seg(k_ptr, k2_ptr, a.seg, j, len_k);
+    const KeySeg<T> gv = key_seg(v_ptr, v2_ptr, a.seg, j, len_k);
+    k_dma.load(tile_src<C::BN, FAR>(gk.base, gk.row0, gk.rows, k_row_bytes, C::ROWB), kd);
+    v_dma.load(tile_src<C::BN, FAR>(gv.base, gv.row0, gv.rows, v_row_bytes, C::ROWB), vd);
   };
 
   auto step = [&](int it, const char* kc, const char* vc, char* kn,

@@ -63,6 +63,13 @@ struct AttnArgs {
   float* sink_part;
   int32_t* sink_count;
   int32_t sink_chunks;  // row chunks per (sequence, kv head)
+  // keys in two row ranges: key rows [0, seg) of k / v / dk / dv, the rest in k2 / v2 / dk2 / dv2
+  // (same strides); seg = INT32_MAX when all keys lie in k / v
+  const void* k2;
+  const void* v2;
+  void* dk2;
+  void* dv2;
+  int32_t seg;
   int32_t avg_keys;  // keys a query row sees on average (host estimate; block shapes hang on it)
   int32_t far;  // a sequence of some streamed tensor spans 2 GiB or more: FAR kernels
   float scale, scale_log2;
@@ -323,6 +330,20 @@ __device__ __forceinline__ TileSrc tile_src(const void* base, int row0, int rows
   } else {
     return {make_rows_rsrc(base, rows, stride_bytes, row_bytes), row0 * stride_bytes};
   }
+}
+
+// Key rows in two ranges (AttnArgs::seg): where the tile of key rows starting at `row0` (never
+// straddling the boundary: seg is a multiple of every tile size) is fetched from.
+template <typename T>
+struct KeySeg {
+  const T* base;
+  int row0, rows;  // first row of the tile inside its range, rows of the range
+};
+template <typename T>
+__device__ __forceinline__ KeySeg<T> key_seg(const T* first, const T* second, int seg, int row0,
+                                             int len_k) {
+  const bool s2 = row0 >= seg;
+  return {s2 ? second : first, s2 ? row0 - seg : row0, s2 ? len_k - seg : min(len_k, seg)};
 }
 
 // Cooperative copy of a [ROWS x D] tile into a swizzled LDS tile with buffer loads that

@@ -152,11 +152,16 @@ void attn_fwd_kernel(const AttnArgs a) {
   k_dma.init(a.k_st[1], tid);
   v_dma.init(a.v_st[1], tid);
   const int k_row_bytes = (int)(a.k_st[1] * 2), v_row_bytes = (int)(a.v_st[1] * 2);
+  // (keys in two row ranges: the second range's tensors, at this batch entry and kv head)
+  const T* k2_ptr = a.k2 ? (const T*)a.k2 + b * a.k_st[0] + hk * a.k_st[2] : k_ptr;
+  const T* v2_ptr = a.v2 ? (const T*)a.v2 + b * a.v_st[0] + hk * a.v_st[2] : v_ptr;
   auto load_k = [&](int it, char* dst) __attribute__((always_inline)) {
-    k_dma.load(tile_src<C::BN, FAR>(k_ptr, tile_of(it) * C::BN, len_k, k_row_bytes, C::ROWB), dst);
+    const KeySeg<T> g = key_seg(k_ptr, k2_ptr, a.seg, tile_of(it) * C::BN, len_k);
+    k_dma.load(tile_src<C::BN, FAR>(g.base, g.row0, g.rows, k_row_bytes, C::ROWB), dst);
   };
   auto load_v = [&](int it, char* dst) __attribute__((always_inline)) {
-    v_dma.load(tile_src<C::BN, FAR>(v_ptr, tile_of(it) * C::BN, len_k, v_row_bytes, C::ROWB), dst);
+    const KeySeg<T> g = key_seg(v_ptr, v2_ptr, a.seg, tile_of(it) * C::BN, len_k);
+    v_dma.load(tile_src<C::BN, FAR>(g.base, g.row0, g.rows, v_row_bytes, C::ROWB), dst);
   };
 
   // ---- pieces of one tile ------------------------------------------------------

@@ -73,7 +73,11 @@ class AttnParams(Structure):
         ("dq_accumulate", c_int32),
         ("addressing", c_int32),
         ("out_accumulate", c_int32),
-        ("reserved_", c_int32),
+        ("seg_rows", c_int32),
+        ("k2", c_void_p),
+        ("v2", c_void_p),
+        ("dk2", c_void_p),
+        ("dv2", c_void_p),
     ]
 
 

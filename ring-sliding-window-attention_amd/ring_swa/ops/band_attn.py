@@ -57,8 +57,30 @@ def _lse_strides(lse: torch.Tensor, packed: bool):
     return (lse.stride(0), lse.stride(1), lse.stride(2))
 
 
+def _same_strides(a, b) -> bool:
+    """Do ``a`` and ``b`` step alike through memory?  (A stride over one element is never used.)"""
+    return all(a.stride(d) == b.stride(d) for d in range(a.dim())
+               if a.shape[d] > 1 and b.shape[d] > 1)
+
+
+def _second_range(p, k, v, second, packed):
+    """Keys in two row ranges: ``(k, v)`` first, then ``second = (k2, v2)`` (dense, same batch,
+    heads, head_dim and strides; ``k.shape[1]`` a multiple of 256)."""
+    k2, v2 = second[0], second[1]
+    assert not packed, "two key ranges in dense mode only"
+    for a, b in ((k, k2), (v, v2)):
+        assert b.dim() == 4 and b.dtype == a.dtype and b.shape[0] == a.shape[0] and \
+            b.shape[2:] == a.shape[2:], "the second key range must match the first but for its rows"
+        assert _same_strides(a, b), "the two key ranges must have the same strides"
+    assert k2.shape == v2.shape and k2.shape[1] > 0
+    assert k.shape[1] % 256 == 0, "the first key range must hold a multiple of 256 rows"
+    p.seqlen_k = k.shape[1] + k2.shape[1]
+    p.seg_rows = k.shape[1]
+    p.k2, p.v2 = k2.data_ptr(), v2.data_ptr()
+
+
 def _params(q, k, v, softmax_scale, window_size, causal, cu_q, cu_k, num_sink,
-            mask_shift=None) -> "_lib.AttnParams":
+            mask_shift=None, second=None) -> "_lib.AttnParams":
     packed = cu_q is not None
     p = _lib.AttnParams()
     p.dtype = _lib.dtype_code(q)
@@ -96,6 +118,8 @@ def _params(q, k, v, softmax_scale, window_size, causal, cu_q, cu_k, num_sink,
     # RSWA_ADDRESSING=far: the kernels that base every tile fetch at the tile's own first row
     # (picked by the library itself once a sequence spans 2 GiB) whatever the sizes
     p.addressing = 1 if os.environ.get("RSWA_ADDRESSING", "") == "far" else 0
+    if second is not None:
+        _second_range(p, k, v, second, packed)
     return p
 
 
@@ -112,8 +136,13 @@ def attn_fwd(
     num_sink: int = 0,
     mask_shift: Optional[int] = None,
     accumulate_into: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+    second: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     """Masked attention forward on the HIP kernel; returns ``(out, lse)``.
+
+    ``second=(k2, v2)``: the keys are the rows of ``k`` followed by the rows of ``k2`` (dense
+    mode; same strides; ``k.shape[1]`` a multiple of 256), taken where they lie -- a ring
+    rank's tail of the previous chunk and its own chunk in one pass, without a concatenation.
 
     ``accumulate_into=(out, lse)``: running partial results of these rows (``out`` in q's
     dtype, ``lse`` fp32, views allowed) that this block is merged into in place, in the
@@ -147,7 +176,7 @@ def attn_fwd(
             lse.fill_(float("-inf"))
             return out, lse
     p = _params(q, k, v, softmax_scale, window_size, causal, cu_seqlens_q, cu_seqlens_k, num_sink,
-                mask_shift)
+                mask_shift, second)
     p.out = out.data_ptr()
     p.out_stride = _lib.i64x3(_strides3(out, packed))
     p.lse = lse.data_ptr()
@@ -172,8 +201,12 @@ def attn_bwd(
     phases: int = 7,
     dq_accumulate: bool = False,
     static_workspace: bool = False,
+    second: Optional[Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]] = None,
 ) -> None:
     """Masked attention backward; overwrites ``dq, dk, dv`` (views are fine).
+
+    ``second=(k2, v2, dk2, dv2)``: keys in two row ranges as in ``attn_fwd``; the gradients of
+    the second range's rows go to ``dk2, dv2`` (shapes and strides of ``k2, v2``).
 
     ``workspace`` (uint8, at least ``bwd_workspace_bytes(q, k, ...)``) may be supplied to avoid the
     per-call scratch allocation, and must be when the phases of one backward are spread
@@ -210,7 +243,16 @@ def attn_bwd(
             dv.zero_()
         return
     p = _params(q, k, v, softmax_scale, window_size, causal, cu_seqlens_q, cu_seqlens_k, num_sink,
-                mask_shift)
+                mask_shift, second)
+    if second is not None:
+        dk2, dv2 = second[2], second[3]
+        _lib.require_device(dk2, dv2)
+        assert dk2.shape == second[0].shape and dv2.shape == second[1].shape
+        assert dk2.dtype == q.dtype and dv2.dtype == q.dtype
+        assert _same_strides(dk2, dk) and _same_strides(dv2, dv), (
+            "dk2 / dv2 must have the strides of dk / dv"
+        )
+        p.dk2, p.dv2 = dk2.data_ptr(), dv2.data_ptr()
     p.dq_accumulate = int(bool(dq_accumulate))
     p.out = o.data_ptr()
     p.out_stride = _lib.i64x3(_strides3(o, packed))
@@ -240,12 +282,14 @@ def attn_bwd(
 
 def bwd_workspace_bytes(q: torch.Tensor, k: torch.Tensor,
                         cu_seqlens_q: Optional[torch.Tensor] = None,
-                        cu_seqlens_k: Optional[torch.Tensor] = None) -> int:
+                        cu_seqlens_k: Optional[torch.Tensor] = None, *,
+                        second_rows: int = 0) -> int:
     """Scratch size of one backward over ``q`` against ``k`` (dense ``[B,S,H,D]`` or packed
     ``[T,H,D]``), as ``rswa_attn_bwd_workspace_bytes`` computes it: two fp32 values per
     (row, q head), plus the partial sums of the dK/dV kernel when the shape makes it deal the
     q heads of a GQA group to several blocks."""
     p = _params(q, k, k, 1.0, (-1, -1), False, cu_seqlens_q, cu_seqlens_k, 0)
+    p.seqlen_k += int(second_rows)  # keys in two row ranges: the rows of the second
     return int(_lib.lib().rswa_attn_bwd_workspace_bytes(p))
 
 

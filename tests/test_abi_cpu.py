@@ -172,3 +172,39 @@ def test_mask_arithmetic_limits_are_refused_or_mapped():
     p.workspace_bytes = 0
     assert L.rswa_attn_bwd(p, None) == -1
     assert b"workspace" in L.rswa_last_error()
+
+
+def test_two_key_ranges_are_checked_before_any_launch():
+    """seg_rows splits the key rows over (k, v) and (k2, v2): dense problems without sink keys,
+    a boundary that is a positive multiple of 256 below seqlen_k, and the second range's
+    tensors present (dk2 / dv2 too for the backward)."""
+    _ensure_built()
+    from ring_swa import _lib
+
+    L = _lib.lib()
+
+    def params(seg=512, **kw):
+        p = _fake_params(1024)
+        p.seg_rows = seg
+        p.k2 = p.v2 = p.dk2 = p.dv2 = 8192
+        for key, val in kw.items():
+            setattr(p, key, val)
+        return p
+
+    for bad in (100, -256, 1024, 1280):
+        assert L.rswa_attn_fwd(params(bad), None) == -2, bad
+        assert b"seg_rows" in L.rswa_last_error()
+    assert L.rswa_attn_fwd(params(num_sink=2), None) == -2
+    assert b"sink" in L.rswa_last_error()
+    assert L.rswa_attn_fwd(params(k2=0), None) == -1
+    assert b"k2" in L.rswa_last_error()
+    assert L.rswa_attn_fwd(params(v2=8), None) == -2       # not 16-byte aligned
+    p = params(dk2=0)
+    p.workspace_bytes = 1 << 30
+    assert L.rswa_attn_bwd(p, None) == -1
+    assert b"dk2" in L.rswa_last_error()
+    # a well-formed pair of ranges passes these checks: the backward goes on to the workspace
+    p = params()
+    p.workspace_bytes = 0
+    assert L.rswa_attn_bwd(p, None) == -1
+    assert b"workspace" in L.rswa_last_error()

@@ -14,10 +14,11 @@ def _inputs(seed, s, hq, hk, d=128):
     return mk(1, s, hq, d), mk(1, s, hk, d), mk(1, s, hk, d), mk(2, 1, s, hk, d), mk(1, s, hq, d)
 
 
-def test_rank_share_step_replays_from_a_graph():
+@pytest.mark.parametrize("w", [300, 256], ids=["two_blocks", "one_band_pass"])
+def test_rank_share_step_replays_from_a_graph(w):
     import ring_swa
 
-    s, hq, hk, w, cp, rank = 512, 4, 2, 300, 4, 2
+    s, hq, hk, cp, rank = 512, 4, 2, 4, 2
     q, k, v, prev, do = _inputs(0, s, hq, hk)
     sq, sk, sv, sprev, sdo = (torch.empty_like(t) for t in (q, k, v, prev, do))
     for dst, src in ((sq, q), (sk, k), (sv, v), (sprev, prev), (sdo, do)):
