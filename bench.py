@@ -30,9 +30,13 @@ PEAK_HBM_GBPS = 8000.0     # MI355X HBM3E
 # HBM bytes per launch (read + written) of the two roofline kernels at the shapes timed below,
 # from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --pmc-pass`, each counter
 # scaled by what it reads for the 1 GiB device copy of that pass (FETCH_SIZE x2.0, WRITE_SIZE
-# x1.0); the summary is profiles/c3_own_chunk_kernels_hbm_traffic_pmc.txt.
-DKDV_HBM_BYTES_PER_LAUNCH = 274.7e6
-MERGE_HBM_BYTES_PER_LAUNCH = 5681.3e6
+# x1.0); the summary is profiles/c3_step_kernels_hbm_traffic_pmc.txt.
+DKDV_HBM_BYTES_PER_LAUNCH = 755.9e6
+MERGE_HBM_BYTES_PER_LAUNCH = 5688.8e6
+# Untimed steps before the W warm-up steps: an idle GPU takes some tens of milliseconds of load to
+# settle its clocks (the first launches of a run take up to a third longer than the later ones), and
+# W = 5 steps are 10 ms.
+SPINUP_STEPS = 40
 
 
 def band_pairs(length: int, w: int) -> int:
@@ -336,7 +340,7 @@ def main():
         print(json.dumps({"pmc_pass": "done", "copy_bytes_each_way": 1 << 30}))
         return
 
-    for _ in range(args.warmup):
+    for _ in range(SPINUP_STEPS + args.warmup):
         step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -354,6 +358,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "spinup_steps": SPINUP_STEPS,
         "ms_per_step": ms,
         "higher_is_better": True,
         "scaling": "weak",
