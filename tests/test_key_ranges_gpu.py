@@ -22,8 +22,11 @@ CASES = [
 ]
 
 
+@pytest.mark.parametrize("addressing", ["near", "far"])
 @pytest.mark.parametrize("case", CASES, ids=[f"c{i}" for i in range(len(CASES))])
-def test_two_key_ranges_equal_concatenated_keys(case):
+def test_two_key_ranges_equal_concatenated_keys(case, addressing, monkeypatch):
+    """(`far`: the kernels that base every tile fetch at the tile's own first row, as the library
+    picks them for tensors beyond 2 GiB.)"""
     from ring_swa.ops import attn_bwd, attn_fwd
     from ring_swa.ops.band_attn import bwd_workspace_bytes
 
@@ -37,11 +40,13 @@ def test_two_key_ranges_equal_concatenated_keys(case):
     kc, vc = torch.cat([k1, k2], 1), torch.cat([v1, v2], 1)
 
     ref_out, ref_lse = attn_fwd(q, kc, vc, None, window, causal)
+    rdq, rdk, rdv = torch.empty_like(q), torch.empty_like(kc), torch.empty_like(vc)
+    attn_bwd(q, kc, vc, ref_out, ref_lse, do, rdq, rdk, rdv, None, window, causal)
+    if addressing == "far":
+        monkeypatch.setenv("RSWA_ADDRESSING", "far")
     out, lse = attn_fwd(q, k1, v1, None, window, causal, second=(k2, v2))
     assert torch.equal(out, ref_out) and torch.equal(lse, ref_lse)
 
-    rdq, rdk, rdv = torch.empty_like(q), torch.empty_like(kc), torch.empty_like(vc)
-    attn_bwd(q, kc, vc, ref_out, ref_lse, do, rdq, rdk, rdv, None, window, causal)
     dq = torch.empty_like(q)
     g = [torch.full_like(t, float("nan")) for t in bufs]
     dk1, dv1, dk2, dv2 = g[0][:, :s1], g[1][:, :s1], g[2][:, :s2], g[3][:, :s2]
