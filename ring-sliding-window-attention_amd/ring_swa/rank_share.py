@@ -303,28 +303,24 @@ def _backward_blocks(q, k, v, prev_kv, out, lse, do, plan, scale, local_cu, ring
 
 
 def _backward_one_pass(q, k, v, prev_kv, out, lse, do, one, scale):
-    """Backward of the one-band forward: one statistics launch, then the dK/dV kernel on the
-    caller's stream and the dQ kernel on the side stream (independent of each other); the
-    gradients of the previous chunk's tail land in their rows of its (zeroed) gradient."""
+    """Backward of the one-band forward: statistics, dQ and dK/dV launches on the caller's
+    stream; the gradients of the previous chunk's tail land in their rows of its (zeroed)
+    gradient.
+
+    One stream: each of the two big launches fills every compute unit by itself (even blocks,
+    many of them), and side by side on two streams they take longer than one after the other
+    (2.01-2.04 against 1.95-1.97 ms per step at 8192-token chunks, window 4096; dQ ahead of
+    dK/dV measured 0.5 % better than the other order)."""
     PREP, DKDV, DQ = 1, 2, 4
     w, kk, vv, _ = one
     s = q.shape[1]
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     dprev = [torch.zeros_like(kv) for kv in prev_kv]
-    second = (k, v, dk, dv)
     dkk, dvv = dprev[0][0][:, s - w:], dprev[0][1][:, s - w:]
     ws = torch.empty(bwd_workspace_bytes(q, kk, second_rows=s), dtype=torch.uint8, device=q.device)
-
-    def run(phases):
+    for phases in (PREP, DQ, DKDV):
         attn_bwd(q, kk, vv, out, lse, do, dq, dkk, dvv, scale, (w, 0), True, workspace=ws,
-                 phases=phases, second=second)
-
-    run(PREP)
-    side = _fork(q.device)
-    with torch.cuda.stream(side):
-        run(DQ)
-    run(DKDV)
-    _join(side, q.device)
+                 phases=phases, second=(k, v, dk, dv))
     return (dq, dk, dv, *dprev)
 
 
