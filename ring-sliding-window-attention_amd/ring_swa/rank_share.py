@@ -211,23 +211,26 @@ def _forward_blocks_accum(q, k, v, prev_kv, plan, scale, local_cu):
 def _one_pass(q, k, v, prev_kv, plan, local_cu):
     """Can the rank's two blocks be computed as ONE band over the previous chunk's tail
     followed by the own chunk?  Yes when the second block is the previous chunk's corner (window
-    shorter than a chunk), its tail holds a multiple of 256 rows and lies like the own chunk in
-    memory: the kernels then take the two row ranges where they are (``second=`` of
-    ``attn_fwd`` / ``attn_bwd``).  Returns ``(window, tail_k, tail_v, tail_rows)`` or None."""
+    shorter than a chunk) and the previous chunk lies like the own chunk in memory: the kernels
+    then take the two row ranges where they are (``second=`` of ``attn_fwd`` / ``attn_bwd``).
+    The tail is the window rounded up to the 256 rows the kernels want the first range to be a
+    multiple of; the rows beyond the window are masked like any key too far back.  Returns
+    ``(window, tail_k, tail_v, tail_rows)`` or None."""
     if local_cu is not None or len(plan) != 2:
         return None
     (_, _, _, (w, _), _), (i1, qs, ks, window1, causal1) = plan
     s = q.shape[1]
     if i1 != 1 or causal1 or window1 != (0, s) or not (0 < w < s):
         return None
-    if (qs.start, qs.stop) != (0, w) or (ks.start, ks.stop) != (s - w, s) or w % 256:
+    tail = -(-w // 256) * 256
+    if (qs.start, qs.stop) != (0, w) or (ks.start, ks.stop) != (s - w, s) or tail > s:
         return None
-    kk, vv = prev_kv[0][0][:, ks], prev_kv[0][1][:, ks]
+    kk, vv = prev_kv[0][0][:, s - tail:], prev_kv[0][1][:, s - tail:]
     # (the kernels apply the first range's strides to both; a stride over one element is unused)
     used = [d for d in range(4) if k.shape[d] > 1]
     if any(kk.stride(d) != k.stride(d) or vv.stride(d) != v.stride(d) for d in used):
         return None
-    return w, kk, vv, w
+    return w, kk, vv, tail
 
 
 def _forward_blocks(q, k, v, prev_kv, plan, scale, local_cu, ring_dtypes):
@@ -312,11 +315,11 @@ def _backward_one_pass(q, k, v, prev_kv, out, lse, do, one, scale):
     (2.01-2.04 against 1.95-1.97 ms per step at 8192-token chunks, window 4096; dQ ahead of
     dK/dV measured 0.5 % better than the other order)."""
     PREP, DKDV, DQ = 1, 2, 4
-    w, kk, vv, _ = one
+    w, kk, vv, tail = one
     s = q.shape[1]
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     dprev = [torch.zeros_like(kv) for kv in prev_kv]
-    dkk, dvv = dprev[0][0][:, s - w:], dprev[0][1][:, s - w:]
+    dkk, dvv = dprev[0][0][:, s - tail:], dprev[0][1][:, s - tail:]
     ws = torch.empty(bwd_workspace_bytes(q, kk, second_rows=s), dtype=torch.uint8, device=q.device)
     for phases in (PREP, DQ, DKDV):
         attn_bwd(q, kk, vv, out, lse, do, dq, dkk, dvv, scale, (w, 0), True, workspace=ws,

@@ -90,10 +90,11 @@ def test_two_key_ranges_match_the_oracle():
     assert _relnorm(dv[:, s - w:], rv[:, s - w:]) <= GRAD_TOL
 
 
-@pytest.mark.parametrize("s_loc,w,cp", [(512, 256, 3), (1024, 768, 2), (768, 512, 2)])
+@pytest.mark.parametrize("s_loc,w,cp", [(512, 256, 3), (1024, 768, 2), (768, 512, 2), (512, 300, 3),
+                                        (1024, 1, 2), (768, 513, 2)])
 def test_rank_share_as_one_band_pass(s_loc, w, cp, monkeypatch):
-    """A rank whose window is shorter than a chunk runs [tail of the previous chunk | own chunk]
-    as one band pass over two key ranges (ring_swa/sliding_window/nonvarlen.py:95-150 runs two
+    """A rank whose window is shorter than a chunk (and, rounded up to 256 rows, no longer than
+    it) runs [tail of the previous chunk | own chunk] as one band pass over two key ranges (ring_swa/sliding_window/nonvarlen.py:95-150 runs two
     blocks and merges).  The shares of all ranks put together must equal the oracle on the whole
     sequence, gradients of the previous chunk included (zero outside the tail), and the step
     must agree with the two-block form of the same step."""
