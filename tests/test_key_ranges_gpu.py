@@ -90,9 +90,9 @@ def test_two_key_ranges_match_the_oracle():
     assert _relnorm(dv[:, s - w:], rv[:, s - w:]) <= GRAD_TOL
 
 
-@pytest.mark.parametrize("s_loc,w,cp", [(512, 256, 3), (1024, 768, 2), (768, 512, 2), (512, 300, 3),
-                                        (1024, 1, 2), (768, 513, 2)])
-def test_rank_share_as_one_band_pass(s_loc, w, cp, monkeypatch):
+@pytest.mark.parametrize("s_loc,w,cp,batch", [(512, 256, 3, 1), (1024, 768, 2, 1), (768, 512, 2, 2),
+                                              (512, 300, 3, 2), (1024, 1, 2, 1), (768, 513, 2, 1)])
+def test_rank_share_as_one_band_pass(s_loc, w, cp, batch, monkeypatch):
     """A rank whose window is shorter than a chunk (and, rounded up to 256 rows, no longer than
     it) runs [tail of the previous chunk | own chunk] as one band pass over two key ranges (ring_swa/sliding_window/nonvarlen.py:95-150 runs two
     blocks and merges).  The shares of all ranks put together must equal the oracle on the whole
@@ -104,8 +104,8 @@ def test_rank_share_as_one_band_pass(s_loc, w, cp, monkeypatch):
     hq, hk, d = 4, 2, 128
     total = s_loc * cp
     g = torch.Generator().manual_seed(21)
-    q, do = (torch.randn(1, total, hq, d, generator=g).bfloat16() for _ in range(2))
-    k, v = (torch.randn(1, total, hk, d, generator=g).bfloat16() for _ in range(2))
+    q, do = (torch.randn(batch, total, hq, d, generator=g).bfloat16() for _ in range(2))
+    k, v = (torch.randn(batch, total, hk, d, generator=g).bfloat16() for _ in range(2))
     ref = O.attention_fwd_bwd(lambda q, k, v: O.sliding_window_attn(q, k, v, w), q, k, v, do)
 
     taken = []
@@ -115,7 +115,7 @@ def test_rank_share_as_one_band_pass(s_loc, w, cp, monkeypatch):
         monkeypatch.setattr(rank_share, "_one_pass", (lambda *a: taken.append(plain(*a)) or taken[-1])
                             if one_pass else (lambda *a: None))
         outs, dqs = [], []
-        dk, dv = torch.zeros(1, total, hk, d), torch.zeros(1, total, hk, d)
+        dk, dv = torch.zeros(batch, total, hk, d), torch.zeros(batch, total, hk, d)
         for r in range(cp):
             sl = slice(r * s_loc, (r + 1) * s_loc)
             qr, kr, vr = (t[:, sl].cuda().requires_grad_() for t in (q, k, v))
