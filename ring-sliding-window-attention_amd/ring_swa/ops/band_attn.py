@@ -73,7 +73,8 @@ def _second_range(p, k, v, second, packed):
             b.shape[2:] == a.shape[2:], "the second key range must match the first but for its rows"
         assert _same_strides(a, b), "the two key ranges must have the same strides"
     assert k2.shape == v2.shape and k2.shape[1] > 0
-    assert k.shape[1] % 256 == 0, "the first key range must hold a multiple of 256 rows"
+    assert k.shape[1] > 0 and k.shape[1] % 256 == 0, (
+        "the first key range must hold a positive multiple of 256 rows")
     p.seqlen_k = k.shape[1] + k2.shape[1]
     p.seg_rows = k.shape[1]
     p.k2, p.v2 = k2.data_ptr(), v2.data_ptr()
