@@ -151,6 +151,7 @@ def attn_fwd(
     ``merge_attn_out``, without the temporaries and the second pass."""
     packed = cu_seqlens_q is not None
     _check_qkv(q, k, v, packed)
+    assert second is None or k.numel() > 0, "two key ranges: the first must not be empty"
     dev = _lib.require_device(q, k, v)
     if softmax_scale is None:
         softmax_scale = q.shape[-1] ** (-0.5)
@@ -219,6 +220,7 @@ def attn_bwd(
     beyond the buffer raise ``NotImplementedError`` and overlapping calls on one GPU race."""
     packed = cu_seqlens_q is not None
     _check_qkv(q, k, v, packed)
+    assert second is None or k.numel() > 0, "two key ranges: the first must not be empty"
     dev = _lib.require_device(q, k, v, o, softmax_lse, do, dq, dk, dv)
     assert o.shape == q.shape and do.shape == q.shape and dq.shape == q.shape
     assert dk.shape == k.shape and dv.shape == v.shape
