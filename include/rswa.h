@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define RSWA_VERSION 1
+#define RSWA_VERSION 2
 
 typedef enum rswa_status {
   RSWA_OK = 0,
@@ -187,6 +187,21 @@ typedef struct rswa_attn_params {
   const void* v2;
   void* dk2;
   void* dv2;
+  /* Backward only.  != 0: dS hand-off.  The dK/dV kernel, which computes P and dS for its own
+   * sums anyway, also stores its 16-bit dS tiles in the workspace, and dq comes from a kernel
+   * that only multiplies them with K (dQ = scale * dS K) instead of computing S = Q K^T and
+   * dP = dO V^T a second time: 12 D multiply-adds per (query, key) pair instead of 14 D for the
+   * whole backward, at the price of 2 bytes per pair written and read once.  The workspace
+   * grows by rswa_attn_bwd_workspace_bytes' account of it (about 2.2 bytes per visible pair and
+   * q head for a window of thousands of keys).  Honoured when the call has no sink keys under a
+   * bounded window, every sequence spans less than 2 GiB (the first addressing form), one
+   * q head's tiles stay below 2 GiB and, with the value 1, the launch is not one of the small
+   * ones whose key tiles are split over several blocks (the value 2 prefers the hand-off to that
+   * split); silently the recomputing route otherwise -- ask rswa_attn_bwd_handoff_active().  With rswa_attn_bwd_phases the DQ phase of this route reads
+   * what the DKDV phase of the same call parameters left in the same workspace, so DKDV must
+   * have run before it.  rswa_attn_bwd_static never uses it.  Same interface replaced:
+   * ring_swa/ops/wrap_flash.py:276-429. */
+  int32_t ds_handoff;
 } rswa_attn_params;
 
 #define RSWA_ADDR_AUTO 0
@@ -233,6 +248,10 @@ int rswa_attn_bwd_static(const rswa_attn_params* p, void* stream);
  * every part (256 keys x head_dim x 2 x 4 bytes each).  The call leaves the counters at zero;
  * nothing in the workspace has to be initialised by the caller. */
 uint64_t rswa_attn_bwd_workspace_bytes(const rswa_attn_params* p);
+
+/* 1 when a backward with these parameters takes the dS hand-off route (ds_handoff != 0 and the
+ * shape is eligible), 0 otherwise. */
+int rswa_attn_bwd_handoff_active(const rswa_attn_params* p);
 
 /* Message of the calling thread's last failed call ("" if none). */
 const char* rswa_last_error(void);

@@ -12,7 +12,21 @@ static uint64_t delta_bytes(const rswa_attn_params* p) {
   return align_up(rows * (uint64_t)p->heads_q * sizeof(float), 256);
 }
 
-BwdLayout bwd_layout(const rswa_attn_params* p, bool allow_split) {
+// Can a backward with these parameters hand dS over?  Not with sink keys under a bounded window
+// (a row tile's key blocks are no longer consecutive), and only in the first addressing form.
+static bool handoff_eligible(const rswa_attn_params* p) {
+  if (p->num_sink > 0 && p->window_left >= 0 && p->window_left < (1 << 28)) return false;
+  if (p->addressing == RSWA_ADDR_FAR) return false;
+  const bool packed = p->cu_seqlens_q != nullptr;
+  const int64_t lim = (1ll << 31) - 65536;
+  const int64_t rq = packed ? p->total_q : p->seqlen_q, rk = packed ? p->total_k : p->seqlen_k;
+  if (rq * p->q_stride[1] * 2 >= lim || rk * p->k_stride[1] * 2 >= lim ||
+      rk * p->v_stride[1] * 2 >= lim || rq * p->dout_stride[1] * 2 >= lim)
+    return false;
+  return true;
+}
+
+BwdLayout bwd_layout(const rswa_attn_params* p, bool allow_split, bool allow_handoff) {
   BwdLayout L{};
   L.nsplit = 1;
   if (!p || p->batch <= 0 || p->heads_q <= 0 || p->heads_kv <= 0 || p->head_dim <= 0) return L;
@@ -24,7 +38,9 @@ BwdLayout bwd_layout(const rswa_attn_params* p, bool allow_split) {
   const int group = p->heads_q / p->heads_kv;
   // Splitting pays when one block per key tile leaves compute units without any work (see
   // kDkvSplitBelow).  The parts of a tile are summed in a fixed order.
-  if (allow_split && group > 1 && blocks > 0 && blocks < kDkvSplitBelow) {
+  // (ds_handoff >= 2: the caller prefers the dS hand-off, which the split kernel does not do)
+  const bool prefer_handoff = allow_handoff && p->ds_handoff >= 2 && handoff_eligible(p);
+  if (allow_split && !prefer_handoff && group > 1 && blocks > 0 && blocks < kDkvSplitBelow) {
     for (int n : {4, 3, 2})
       if (group % n == 0) {
         L.nsplit = n;
@@ -50,10 +66,37 @@ BwdLayout bwd_layout(const rswa_attn_params* p, bool allow_split) {
   L.sink_off = L.part_off + (uint64_t)split_units * L.nsplit * per_unit;
   L.total_bytes = L.sink_off + (uint64_t)sink_units * L.sink_chunks * p->num_sink * 2 * p->head_dim *
                                    sizeof(float);
+  // dS hand-off: one 4 KiB unit per (q head, 32-row tile slot, 256-key block modulo nkb, 64-key
+  // group).  A row tile sees keys [i0 + shift - left, i0 + 31 + shift + right]: left + right + 32
+  // consecutive keys, which touch at most (left + right + 31) / 256 + 2 blocks of 256, and never
+  // more than a sequence has.
+  // (Launches whose key tiles are split over several blocks are small ones; they keep the
+  // recomputing route: the split kernel has no registers left for the hand-off.)
+  if (allow_handoff && p->ds_handoff && L.nsplit == 1 && handoff_eligible(p)) {
+    const int64_t rows_q = packed ? p->total_q : (int64_t)p->batch * p->seqlen_q;
+    const int64_t blocks_seq = (rows_k + kDkvKeysPerBlock - 1) / kDkvKeysPerBlock;  // rows_k: one sequence's bound
+    int64_t nkb = blocks_seq;
+    const bool causal = p->causal != 0;
+    const int64_t wl = p->window_left, wr = causal ? 0 : p->window_right;
+    if (wl >= 0 && wr >= 0 && wl < (1 << 28) && wr < (1 << 28))
+      nkb = std::min<int64_t>(nkb, (wl + wr + 31) / kDkvKeysPerBlock + 2);
+    nkb = std::max<int64_t>(nkb, 1);
+    const int64_t slots = packed ? (rows_q + 31) / 32 + p->batch
+                                 : (int64_t)p->batch * ((p->seqlen_q + 31) / 32);
+    const uint64_t head_bytes = (uint64_t)slots * nkb * kDsBlockBytes;
+    // (the dK/dV kernel addresses the units of a GQA group's heads through 32-bit offsets)
+    if (rows_q > 0 && rows_k > 0 && head_bytes * (uint64_t)group < 0x7ff00000ull) {
+      L.ds_nkb = (int)nkb;
+      L.ds_slots = (int)slots;
+      L.ds_off = align_up(L.total_bytes, 4096);
+      L.ds_bytes = head_bytes * (uint64_t)p->heads_q;
+      L.total_bytes = L.ds_off + L.ds_bytes;
+    }
+  }
   return L;
 }
 
-uint64_t bwd_workspace_bytes(const rswa_attn_params* p) { return bwd_layout(p, true).total_bytes; }
+uint64_t bwd_workspace_bytes(const rswa_attn_params* p) { return bwd_layout(p, true, true).total_bytes; }
 
 static bool rows_aligned(const void* ptr, const int64_t* st) {
   if (((uintptr_t)ptr) % 16) return false;
@@ -62,7 +105,8 @@ static bool rows_aligned(const void* ptr, const int64_t* st) {
   return true;
 }
 
-int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a, bool allow_split) {
+int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a, bool allow_split,
+              bool allow_handoff) {
   RSWA_REQUIRE(p != nullptr, RSWA_ERR_INVALID, "attn: null params");
   RSWA_REQUIRE(p->dtype == RSWA_BF16 || p->dtype == RSWA_F16, RSWA_ERR_UNSUPPORTED,
                "attn: dtype %d (only bf16 and fp16)", p->dtype);
@@ -149,6 +193,9 @@ int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a, bool allow_
   a.sink_part = nullptr;
   a.sink_count = nullptr;
   a.sink_chunks = 0;
+  a.ds = nullptr;
+  a.ds_nkb = 0;
+  a.ds_slots = 0;
   a.cu_q = p->cu_seqlens_q;
   a.cu_k = p->cu_seqlens_k;
   for (int i = 0; i < 3; i++) {
@@ -226,7 +273,7 @@ int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a, bool allow_
                  RSWA_ERR_UNSUPPORTED, "attn_bwd: dout/dq/dk/dv rows must start 16-byte aligned");
     RSWA_REQUIRE(p->dout_stride[1] >= 0 && p->dout_stride[1] * 2 < ((1ll << 31) - 65536) / kMaxTileRows,
                  RSWA_ERR_UNSUPPORTED, "attn_bwd: row stride of dout is negative or too large");
-    const BwdLayout L = bwd_layout(p, allow_split);
+    const BwdLayout L = bwd_layout(p, allow_split, allow_handoff);
     const uint64_t need = L.total_bytes;
     RSWA_REQUIRE(p->workspace != nullptr || need == 0, RSWA_ERR_INVALID,
                  "attn_bwd: null workspace");
@@ -244,6 +291,11 @@ int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a, bool allow_
     a.sink_chunks = L.sink_chunks;
     a.sink_part = L.sink_chunks ? (float*)((char*)p->workspace + L.sink_off) : nullptr;
     a.sink_count = a.dkv_count + L.sink_count_index;
+    if (L.ds_bytes) {
+      a.ds = (char*)p->workspace + L.ds_off;
+      a.ds_nkb = L.ds_nkb;
+      a.ds_slots = L.ds_slots;
+    }
     // one load reaches from a row's lse2 to its delta, one array further on
     RSWA_REQUIRE(delta_bytes(p) < (1ull << 31) - 65536, RSWA_ERR_UNSUPPORTED,
                  "attn_bwd: rows * heads_q = %lld: each statistics array must stay below 2 GiB "
@@ -257,4 +309,8 @@ int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a, bool allow_
 
 extern "C" uint64_t rswa_attn_bwd_workspace_bytes(const rswa_attn_params* p) {
   return rswa::bwd_workspace_bytes(p);
+}
+
+extern "C" int rswa_attn_bwd_handoff_active(const rswa_attn_params* p) {
+  return rswa::bwd_layout(p, true, true).ds_bytes != 0;
 }

@@ -69,8 +69,9 @@ struct DkvCfg {
   static constexpr int Q_TILE = BM * ROWB;
 };
 
-template <typename T, int D, bool SPLIT, bool FAR>
+template <typename T, int D, bool SPLIT, bool FAR, bool HAND>
 __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
+  static_assert(!(HAND && FAR), "dS hand-off in the first addressing form only");
   using C = DkvCfg<D>;
   using M = Mma<T>;
   using V8 = typename M::V8;
@@ -213,6 +214,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
     int qt, i0;
     const T *q_head, *do_head;
     int stat_row;  // index of row 0 of this head in the statistics arrays
+    int ds;        // HAND: byte offset of this wave's dS unit of the tile (from ds_first)
   };
   const int i_first = qt_lo * C::BM;
   // Every head's walk over the n_qt query tiles starts at tile qt_start and wraps around,
@@ -228,6 +230,26 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   nxt.q_head = q_base + (int64_t)h_first * a.q_st[2];
   nxt.do_head = do_base + (int64_t)h_first * a.do_st[2];
   nxt.stat_row = (int)(h_first * a.rows_q + ws_row0);
+  // dS hand-off: unit of (q head h, row tile qt of the sequence, this block's keys, this wave) at
+  //   ds + (((h ds_slots + slot0 + qt) ds_nkb + kt % ds_nkb) 4 + wave) 4 KiB
+  // -- per step one row of ds_nkb blocks further, per head ds_slots rows further.  The units
+  // of the block's heads are addressed as 32-bit offsets from that of its first head's first
+  // tile, through a buffer resource that ends with the last head's rows: an offset beyond it
+  // (kDsNowhere) makes the hardware drop the store.
+  const int ds_row_bytes = HAND ? a.ds_nkb * kDsBlockBytes : 0;
+  const int ds_head_bytes = HAND ? a.ds_slots * ds_row_bytes : 0;  // (host: group x this < 2 GiB)
+  constexpr int kDsNowhere = 0x7ff00000;
+  const int64_t ds_slot0 = a.cu_q ? (s.q_row0 >> 5) + b : (int64_t)b * ((a.seqlen_q + 31) >> 5);
+  const int64_t ds_first = HAND ? (int64_t)h_first * ds_head_bytes + (ds_slot0 + qt_lo) * ds_row_bytes +
+                                      (kt % max(a.ds_nkb, 1)) * kDsBlockBytes + wave * kDsUnitBytes
+                                : 0;
+  const __amdgpu_buffer_rsrc_t ds_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      a.ds + ds_first, 0,
+      HAND ? (int)min((int64_t)hpu * ds_head_bytes, (int64_t)a.heads_q * ds_head_bytes - ds_first) : 0,
+      0x00020000);
+  int ds_head_off = 0;  // of the head the cursor is on
+  nxt.ds = qt_start * ds_row_bytes;
+  [[maybe_unused]] int cur_ds = nxt.ds;  // the unit of the tile being computed
   // The next tile is fetched by NPART instructions per wave (statistics, Q, dO), issued
   // one at a time between the first MFMAs of a step; advance() then moves the cursor on.
   constexpr int NQD = TileDma<D, C::BM, C::THREADS>::N;
@@ -255,9 +277,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   auto advance = [&]() __attribute__((always_inline)) {
     nxt.qt++;
     nxt.i0 += C::BM;
+    if constexpr (HAND) nxt.ds += ds_row_bytes;
     if (nxt.qt == n_qt) {
       nxt.qt = 0;
       nxt.i0 = i_first;
+      if constexpr (HAND) nxt.ds = ds_head_off;
     }
     if (--nxt_left == 0) {
       nxt_left = n_qt;
@@ -266,6 +290,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
       nxt.q_head += a.q_st[2];
       nxt.do_head += a.do_st[2];
       nxt.stat_row += (int)a.rows_q;
+      if constexpr (HAND) {
+        ds_head_off += ds_head_bytes;
+        nxt.ds = ds_head_off + qt_start * ds_row_bytes;
+      }
     }
   };
 
@@ -278,6 +306,31 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
 
 
   int cur_i0 = i_first + qt_start * C::BM;  // first row of the tile being computed
+  // byte of a lane's 16 in a 1 KiB piece of a dS unit: [key l32][query group g]
+  const int ds_lane = l32 * 32 + g * 16;
+  // dS of a step, packed to 16 bits as the operand of its dK MFMAs.  HAND: the four groups also
+  // go to the step's dS unit -- under the first MFMAs of the NEXT step (stores issued late in
+  // their own step would still be on their way at its end, and the wait for the tile loads
+  // there waits for every vector memory operation of the wave: that cost a fifth of the
+  // kernel).  ds_pend = where they go: the unit of the last computed step, or nowhere.
+  [[maybe_unused]] V8 ds_carry[KB][2];
+  [[maybe_unused]] int ds_pend = kDsNowhere;
+  auto store_ds = [&](int pc, int voff) __attribute__((always_inline)) {
+    // piece [key block][query half] of the unit, 1 KiB per wave instruction: a key's 32 bytes
+    // side by side ([query group g][rows 16 ks2 + 4 g .., 16 ks2 + 8 + 4 g ..])
+    u32x4 bits;
+    __builtin_memcpy(&bits, &ds_carry[pc >> 1][pc & 1], 16);
+    // (aux 2 = non-temporal: the tiles are read once, by another kernel, much later; measured
+    // 6 % faster than plain stores on a 2.4 GB hand-off)
+    __builtin_amdgcn_raw_buffer_store_b128(bits, ds_rsrc, voff + pc * 1024, ds_pend, 2);
+  };
+  // (the lane's offset, opaque to the optimiser: or it keeps the four sums voff + pc * 1024 in
+  // registers across the walk instead of using the instruction's immediate offset)
+  auto ds_voff = [&]() __attribute__((always_inline)) {
+    int v = ds_lane;
+    asm volatile("" : "+v"(v));
+    return v;
+  };
   // For which first rows i0 of a 32-row tile does any (query, key of this wave) pair survive
   // the mask (need_*), and for which is no pair masked (full_*)?  With
   // i1 = min(i0 + 32, len_q) - 1 and the wave's keys jw0 .. jw1 the conditions
@@ -297,6 +350,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
                   float* stn) __attribute__((always_inline)) {
     const int i0 = cur_i0;
     cur_i0 = nxt.i0;  // the tile fetched now is the next step's
+    [[maybe_unused]] const int ds_unit = cur_ds;
+    cur_ds = nxt.ds;
     const bool has_next = it + 1 < n_iter;
     const float* lse_lds = stc;
     const float* delta_lds = stc + C::BM;
@@ -305,6 +360,14 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
 #pragma unroll
       for (int part = 0; part < NPART; part++) load_part(part, qn, don, stn);
       if (it + 2 < n_iter) advance();
+    }
+    if constexpr (HAND) {
+      if (!needed) {
+        const int voff = ds_voff();
+#pragma unroll
+        for (int pc = 0; pc < 2 * KB; pc++) store_ds(pc, voff);
+        ds_pend = kDsNowhere;
+      }
     }
     if (needed) {
       const bool full = i0 >= full_lo && i0 <= full_hi;
@@ -343,7 +406,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
       // into the second key block's accumulator: the first block's chain takes it as a separate
       // start operand, the second block's chain then accumulates in place
       f32x4 l4[4];   // -lse2 of the rows
-      V8 pb[KB][2], dsb[KB][2];
+      V8 pb[KB][2], ds_step[KB][2];
+      V8(&dsb)[KB][2] = *[&]() __attribute__((always_inline)) {
+        if constexpr (HAND) return &ds_carry;  // lives on into the next step
+        else return &ds_step;
+      }();
       // vector work in 2 KB chunks of four rows: chunk order lets the packed operands of
       // the first k-step be complete first
       auto chunk_of = [](int c, int& kb, int& i4) __attribute__((always_inline)) {
@@ -375,6 +442,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
         if (i4 & 1) dsb[kb][i4 >> 1] = M::pack(dsk[kb]);
       };
 
+      [[maybe_unused]] int ds_voff_step = 0;
+      if constexpr (HAND) ds_voff_step = ds_voff();
       static_for<AH>([&](auto fc) __attribute__((always_inline)) { fetch(fc); });
       fence();
       static_for<4 * NG>([&](auto mc) __attribute__((always_inline)) {
@@ -384,6 +453,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
         // (after the last tile the cursor still names it: its rows are fetched once more, into
         // the idle buffers, rather than branching around every load)
         if constexpr (m < NPART) load_part(m, qn, don, stn);
+        if constexpr (HAND && m < 2 * KB) {
+          store_ds(m, ds_voff_step);
+          if constexpr (m == 2 * KB - 1) ds_pend = ds_unit;
+        }
         // row statistics: -delta early in S (the dP chains start from it), -lse2 at its end
         if constexpr (m >= 4 && m < 8) {
           const f32x4 t4 = *(const f32x4*)(delta_lds + 8 * (m - 4) + 4 * g);
@@ -451,6 +524,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   for (int it = 0; it < n_iter; it += 2) {
     step(it, q_s0, do_s0, st_s0, q_s1, do_s1, st_s1);
     if (it + 1 < n_iter) step(it + 1, q_s1, do_s1, st_s1, q_s0, do_s0, st_s0);
+  }
+  if constexpr (HAND) {  // the last computed step's dS
+    const int voff = ds_voff();
+#pragma unroll
+    for (int pc = 0; pc < 2 * KB; pc++) store_ds(pc, voff);
   }
 
   // ---- write dK, dV (C layout: lane = key, regs = d) -----------------------------------
@@ -1099,6 +1177,261 @@ void attn_bwd_dq_kernel(const AttnArgs a) {
 }
 
 // ============================================================================
+// dQ from handed-over dS
+// ============================================================================
+// The dK/dV kernel of the hand-off route leaves, per (q head, 32-row query tile, 64-key group),
+// the 16-bit dS values it computed (zero where the mask hides a pair): a 4 KiB unit of four
+// 1 KiB pieces [32-key block kb][query half ks2], a piece holding for each of its 32 keys 32
+// bytes: the key's dS for queries 16 ks2 + {0..3, 8..11} and then 16 ks2 + {4..7, 12..15}.  This
+// kernel only computes dQ^T += K^T dS^T (2 D multiply-adds per pair, against the 6 D of the
+// kernel that recomputes S and dP), so it is bound by reading those units once: it keeps two
+// stages of them in flight while it works on a third.
+//
+// Block = 4 waves; a wave owns 64 query rows (two 32-row tiles) of one q head: the 4 waves are
+// 4 / 2 / 1 q heads of a GQA group on the same 64 / 128 / 256 rows, sharing each 64-key K tile.
+// Per 16 keys and wave: A = K^T (32 d x 16 keys, transposing reads of the K tile), B = dS^T
+// (16 keys x 32 queries, transposing reads of the unit: the 16-lane groups of such a read take
+// 4 keys x 16 queries, which is 128 consecutive bytes of a piece), C = dQ^T (lane = query).
+template <int D>
+struct DqDsCfg {
+  static constexpr int BN = 64;   // keys per stage
+  static constexpr int NST = 3;   // stages held in LDS
+  static constexpr int ROWB = D * 2;
+  static constexpr int CPR = D / 8;
+  static constexpr int DBLK = D / 32;
+  static constexpr int K_TILE = BN * ROWB;
+  // LDS image of a unit: piece (kb, ks2) at kb KBLK + ks2 PIECE1 -- 128 bytes between the two
+  // query halves, which the two halves of a half-wave read together, put them on different banks
+  static constexpr int PIECE1 = 1024 + 128;
+  static constexpr int KBLK = 2048 + 256;
+  static constexpr int UNIT_LDS = 2 * KBLK;
+  static constexpr int WAVE_LDS = 2 * UNIT_LDS;
+  static constexpr int O_STRIDE = D * 2 + 16;
+  static_assert(WAVE_LDS >= 32 * O_STRIDE, "a wave's epilogue staging fits its dS buffers of a stage");
+  static constexpr int NKD = BN * CPR / 256;  // K tile load instructions per wave and stage
+  static constexpr int NLD = NKD + 8;         // ... and all loads
+};
+
+template <typename T, int D>
+__global__ __launch_bounds__(256) void attn_bwd_dq_ds_kernel(const AttnArgs a) {
+  using C = DqDsCfg<D>;
+  using M = Mma<T>;
+  using V8 = typename M::V8;
+  constexpr int DB = C::DBLK;
+  __shared__ __attribute__((aligned(1024))) char k_s0[C::K_TILE];
+  __shared__ __attribute__((aligned(1024))) char k_s1[C::K_TILE];
+  __shared__ __attribute__((aligned(1024))) char k_s2[C::K_TILE];
+  __shared__ __attribute__((aligned(1024))) char ds_s0[4 * C::WAVE_LDS];
+  __shared__ __attribute__((aligned(1024))) char ds_s1[4 * C::WAVE_LDS];
+  __shared__ __attribute__((aligned(1024))) char ds_s2[4 * C::WAVE_LDS];
+
+  const int wid = logical_block_id(a.n_work);
+  if (wid < 0) return;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c32 = lane & 31;  // query column of a tile
+  const int gg = lane >> 5;   // k half
+  const int i16 = lane & 15;
+
+  // heads per block: 4, 2 or 1 (the rest of the waves go to further 64-row units)
+  const int hsh = (a.group & 3) == 0 ? 2 : (a.group & 1) == 0 ? 1 : 0;
+  const int units = a.group >> hsh;
+  const int bm_log2 = 8 - hsh;  // 64 rows x (4 >> hsh) units
+  const int bm = 1 << bm_log2;
+  const int hu = wid % units;
+  int rest = wid / units;
+  const int slot = a.rev_q ? a.n_tile - 1 - rest % a.n_tile : rest % a.n_tile;
+  rest /= a.n_tile;
+  const int hk = rest % a.heads_kv;
+  const int hq = hk * a.group + (hu << hsh) + (wave & ((1 << hsh) - 1));
+  SeqInfo s;
+  int qt;
+  if (a.cu_q) {
+    if (!locate_packed(a, slot, bm_log2, false, s, qt)) return;
+  } else {
+    s.batch_idx = rest / a.heads_kv;
+    s.q_row0 = s.k_row0 = 0;
+    s.len_q = a.seqlen_q;
+    s.len_k = a.seqlen_k;
+    qt = slot;
+  }
+  const int b = s.batch_idx;
+  const int len_q = s.len_q, len_k = s.len_k;
+  const int i0 = qt << bm_log2;
+  if (i0 >= len_q) return;
+
+  const T* k_ptr = (const T*)a.k + b * a.k_st[0] + s.k_row0 * a.k_st[1] + hk * a.k_st[2];
+  const T* k2_ptr = a.k2 ? (const T*)a.k2 + b * a.k_st[0] + hk * a.k_st[2] : k_ptr;
+  T* dq_ptr = (T*)a.dq + b * a.dq_st[0] + s.q_row0 * a.dq_st[1] + hq * a.dq_st[2];
+
+  // ---- key stages of the block (64 keys each): those any of its rows can see -------------
+  const int i_last = min(i0 + bm, len_q) - 1;
+  const int lo_blk = row_bounds(a, i0, len_q, len_k).lo;
+  const int hi_blk = row_bounds(a, i_last, len_q, len_k).hi;
+  const int t_lo = lo_blk / C::BN;
+  const int n_st = hi_blk >= lo_blk ? hi_blk / C::BN - t_lo + 1 : 0;
+
+  // ---- this wave's two row tiles, and for which stages j0 the dK/dV kernel wrote their unit:
+  // its wave (keys j0 .. j0 + 63) computed tile i iff some pair of the two survives the mask,
+  //   i < len_q, j0 < len_k, j0 <= min(i + 31, len_q - 1) + shift + right,
+  //   min(j0 + 63, len_k - 1) >= i + shift - left
+  const int r0 = i0 + ((wave >> hsh) << 6);
+  const int shift = a.shift_explicit ? a.shift_val : len_k - len_q;
+  constexpr int kInf = 1 << 30;
+  int jmin[2], jmax[2];
+#pragma unroll
+  for (int t = 0; t < 2; t++) {
+    const int it = r0 + 32 * t;
+    jmax[t] = (a.wr < 0) ? len_k - 1 : min(len_k - 1, min(it + 31, len_q - 1) + shift + a.wr);
+    jmin[t] = (a.wl < 0) ? -kInf : it + shift - a.wl - (C::BN - 1);
+    if (it >= len_q || (a.wl >= 0 && it + shift - a.wl > len_k - 1)) jmax[t] = -kInf - 1;
+  }
+
+  // ---- the wave's dS units: rows of ds_nkb blocks of 4 units per (head, tile slot) ---------
+  const int ds_row_bytes = a.ds_nkb * kDsBlockBytes;
+  const int64_t ds_head_bytes = (int64_t)a.ds_slots * ds_row_bytes;
+  const int64_t slot0 = a.cu_q ? (s.q_row0 >> 5) + b : (int64_t)b * ((a.seqlen_q + 31) >> 5);
+  const int64_t ds_off = hq * ds_head_bytes + (slot0 + (r0 >> 5)) * ds_row_bytes;
+  const int64_t ds_left = (int64_t)a.heads_q * ds_head_bytes - ds_off;  // bytes up to the buffer's end
+  const int ds_span = r0 < len_q ? (int)min((int64_t)2 * ds_row_bytes, ds_left) : 0;
+  const __amdgpu_buffer_rsrc_t ds_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void*)(a.ds + (ds_span > 0 ? ds_off : 0)), 0, ds_span, 0x00020000);
+  const int ds_voff = lane * 16;
+
+  TileDma<D, C::BN, 256> k_dma;
+  k_dma.init(a.k_st[1], tid);
+  const int k_row_bytes = (int)(a.k_st[1] * 2);
+
+  // load cursor: the stage fetched next
+  int ld_j = t_lo * C::BN;
+  int ld_kb = (ld_j >> 8) % a.ds_nkb;
+  auto load_stage = [&](char* kd, char* dsd) __attribute__((always_inline)) {
+    const KeySeg<T> gk = key_seg(k_ptr, k2_ptr, a.seg, ld_j, len_k);
+    k_dma.load(tile_src<C::BN, false>(gk.base, gk.row0, gk.rows, k_row_bytes, C::ROWB), kd);
+    const int soff = ld_kb * kDsBlockBytes + ((ld_j >> 6) & 3) * kDsUnitBytes;
+    char* dst = dsd + wave * C::WAVE_LDS;
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+      for (int pc = 0; pc < 4; pc++)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            ds_rsrc, (lds_void_t*)(dst + t * C::UNIT_LDS + (pc >> 1) * C::KBLK + (pc & 1) * C::PIECE1), 16,
+            ds_voff, t * ds_row_bytes + soff + pc * 1024, 0, 0);
+    ld_j += C::BN;
+    if ((ld_j & 255) == 0) ld_kb = ld_kb + 1 == a.ds_nkb ? 0 : ld_kb + 1;
+  };
+
+  // ---- lane-constant LDS offsets ------------------------------------------------------------
+  // transposing reads of K: rows 16 s + 8 gg + (i16 >> 2) (+ 4), chunk 4 db + 2 (c32 / 16) +
+  // ((i16 & 3) >> 1), second half of the chunk for odd i16
+  //   offset = (kt_row{0,1} ^ (db << 6)) + s * 16 * ROWB
+  const int krow = 8 * gg + (i16 >> 2);
+  const int kch = 2 * (c32 >> 4) + ((i16 & 3) >> 1);
+  const int kt_row0 = krow * C::ROWB + ((kch ^ swz_f<C::CPR>(krow)) << 4) + (i16 & 1) * 8;
+  const int kt_row1 = (krow + 4) * C::ROWB + ((kch ^ swz_f<C::CPR>(krow + 4)) << 4) + (i16 & 1) * 8;
+  // transposing reads of a dS unit: key 16 (s & 1) + 8 gg + (i16 >> 2) (+ 4) of block s >> 1,
+  // queries 16 (c32 / 16) + 4 (i16 & 3) ..: byte (i16 & 1) 16 + ((i16 >> 1) & 1) 8 of the key's 32
+  const int ds_row = (c32 >> 4) * C::PIECE1 + krow * 32 + (i16 & 1) * 16 + ((i16 >> 1) & 1) * 8;
+
+  f32x16 acc[2][DB];
+#pragma unroll
+  for (int t = 0; t < 2; t++)
+#pragma unroll
+    for (int d = 0; d < DB; d++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) acc[t][d][i] = 0.f;
+
+  int cur_j = t_lo * C::BN;
+  auto stage = [&](int it, const char* kc, const char* dsc, char* kn, char* dsn)
+      __attribute__((always_inline)) {
+    // this wave's loads of the stage have landed (those of the next one may still fly) ...
+    if (it + 1 < n_st) {
+      wait_vmem_but<C::NLD>();
+    } else {
+      wait_vmem_but<0>();
+    }
+    // ... and everybody's: the K tile is complete, and nobody reads the buffers of the stage
+    // before this one any more, which the loads of the stage after the next now overwrite
+    lds_barrier();
+    if (it + 2 < n_st) load_stage(kn, dsn);
+    const int j0 = cur_j;
+    cur_j += C::BN;
+    const bool n0 = j0 >= jmin[0] && j0 <= jmax[0];
+    const bool n1 = j0 >= jmin[1] && j0 <= jmax[1];
+    if (!(n0 || n1)) return;
+    const char* dsw = dsc + wave * C::WAVE_LDS + ds_row;
+    auto body = [&](auto c0, auto c1) __attribute__((always_inline)) {
+      constexpr bool T0 = decltype(c0)::value, T1 = decltype(c1)::value;
+#pragma unroll
+      for (int sl = 0; sl < 4; sl++) {
+        V8 kt[DB];
+#pragma unroll
+        for (int d = 0; d < DB; d++)
+          kt[d] = tr_pair<V8>(kc + (kt_row0 ^ (d << 6)) + sl * 16 * C::ROWB,
+                              kc + (kt_row1 ^ (d << 6)) + sl * 16 * C::ROWB);
+        const int uo = (sl >> 1) * C::KBLK + (sl & 1) * 512;
+        if constexpr (T0) {
+          const V8 dsf = tr_pair<V8>(dsw + uo, dsw + uo + 128);
+#pragma unroll
+          for (int d = 0; d < DB; d++) acc[0][d] = M::mfma32(kt[d], dsf, acc[0][d]);
+        }
+        if constexpr (T1) {
+          const V8 dsf = tr_pair<V8>(dsw + C::UNIT_LDS + uo, dsw + C::UNIT_LDS + uo + 128);
+#pragma unroll
+          for (int d = 0; d < DB; d++) acc[1][d] = M::mfma32(kt[d], dsf, acc[1][d]);
+        }
+      }
+    };
+    if (n0 && n1) body(std::true_type{}, std::true_type{});
+    else if (n0) body(std::true_type{}, std::false_type{});
+    else body(std::false_type{}, std::true_type{});
+  };
+
+  if (n_st > 0) load_stage(k_s0, ds_s0);
+  if (n_st > 1) load_stage(k_s1, ds_s1);
+  for (int it = 0; it < n_st; it += 3) {
+    stage(it, k_s0, ds_s0, k_s2, ds_s2);
+    if (it + 1 < n_st) stage(it + 1, k_s1, ds_s1, k_s0, ds_s0);
+    if (it + 2 < n_st) stage(it + 2, k_s2, ds_s2, k_s1, ds_s1);
+  }
+
+  // ---- epilogue: dq = scale * acc, a tile at a time through the wave's own LDS ----------------
+  // element i of acc[t][d] is dQ[query 32 t + c32][32 d + 8 (i / 4) + 4 gg + i % 4]
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  char* stg = ds_s0 + wave * C::WAVE_LDS;
+#pragma unroll
+  for (int t = 0; t < 2; t++) {
+#pragma unroll
+    for (int d = 0; d < DB; d++)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; i4++)
+        *(typename M::V4*)(stg + c32 * C::O_STRIDE + (32 * d + 8 * i4 + 4 * gg) * 2) =
+            M::pack4(acc[t][d][4 * i4] * a.scale, acc[t][d][4 * i4 + 1] * a.scale,
+                     acc[t][d][4 * i4 + 2] * a.scale, acc[t][d][4 * i4 + 3] * a.scale);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int n = 0; n < 32 * C::CPR / 64; n++) {
+      const int cc = lane + n * 64;
+      const int row = cc / C::CPR, col = (cc % C::CPR) * 8;
+      V8 val = *(const V8*)(stg + row * C::O_STRIDE + col * 2);
+      if (r0 + 32 * t + row < len_q) {
+        T* dst = dq_ptr + (int64_t)(r0 + 32 * t + row) * a.dq_st[1] + col;
+        if (a.dq_accumulate) {
+          const V8 old = *(const V8*)dst;
+          float sum[8];
+#pragma unroll
+          for (int j = 0; j < 8; j++) sum[j] = (float)old[j] + (float)val[j];
+          val = M::pack(sum);
+        }
+        *(V8*)dst = val;
+      }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  }
+}
+
+// ============================================================================
 // row statistics, stored negated: -delta = -sum_d dO * O and -lse2 = -lse * log2(e) (empty
 // rows: -inf, so that P = exp2(S*c - lse2) is zero).  One 16-lane (D=128) or 8-lane (D=64) group per
 // (row, head).
@@ -1160,10 +1493,12 @@ __global__ __launch_bounds__(256) void attn_bwd_prep_kernel(const AttnArgs a) {
 // Explicit instantiations: with implicit instantiation alone this hipcc emits the host
 // launch stubs of only some of the variants.
 #define RSWA_INSTANTIATE(T, D)                                              \
-  template __global__ void attn_bwd_dkdv_kernel<T, D, false, false>(const AttnArgs); \
-  template __global__ void attn_bwd_dkdv_kernel<T, D, true, false>(const AttnArgs);  \
-  template __global__ void attn_bwd_dkdv_kernel<T, D, false, true>(const AttnArgs);  \
-  template __global__ void attn_bwd_dkdv_kernel<T, D, true, true>(const AttnArgs);   \
+  template __global__ void attn_bwd_dkdv_kernel<T, D, false, false, false>(const AttnArgs); \
+  template __global__ void attn_bwd_dkdv_kernel<T, D, true, false, false>(const AttnArgs);  \
+  template __global__ void attn_bwd_dkdv_kernel<T, D, false, true, false>(const AttnArgs);  \
+  template __global__ void attn_bwd_dkdv_kernel<T, D, true, true, false>(const AttnArgs);   \
+  template __global__ void attn_bwd_dkdv_kernel<T, D, false, false, true>(const AttnArgs);  \
+  template __global__ void attn_bwd_dq_ds_kernel<T, D>(const AttnArgs);                     \
   template __global__ void attn_bwd_dq_kernel<T, D, false, 8>(const AttnArgs);       \
   template __global__ void attn_bwd_dq_kernel<T, D, true, 8>(const AttnArgs);        \
   template __global__ void attn_bwd_dq_kernel<T, D, false, 4>(const AttnArgs);       \
@@ -1199,12 +1534,14 @@ int launch_bwd(AttnArgs& a, hipStream_t stream, int phases) {
     if (a.n_work > 0) {
       clear_launch_error();
       const dim3 grid(padded_grid(a.n_work)), block(C::THREADS);
-      if (a.nsplit > 1) {
-        if (a.far) hipLaunchKernelGGL((attn_bwd_dkdv_kernel<T, D, true, true>), grid, block, 0, stream, a);
-        else hipLaunchKernelGGL((attn_bwd_dkdv_kernel<T, D, true, false>), grid, block, 0, stream, a);
+      if (a.ds) {  // (never with a.far or a.nsplit > 1: see bwd_layout)
+        hipLaunchKernelGGL((attn_bwd_dkdv_kernel<T, D, false, false, true>), grid, block, 0, stream, a);
+      } else if (a.nsplit > 1) {
+        if (a.far) hipLaunchKernelGGL((attn_bwd_dkdv_kernel<T, D, true, true, false>), grid, block, 0, stream, a);
+        else hipLaunchKernelGGL((attn_bwd_dkdv_kernel<T, D, true, false, false>), grid, block, 0, stream, a);
       } else {
-        if (a.far) hipLaunchKernelGGL((attn_bwd_dkdv_kernel<T, D, false, true>), grid, block, 0, stream, a);
-        else hipLaunchKernelGGL((attn_bwd_dkdv_kernel<T, D, false, false>), grid, block, 0, stream, a);
+        if (a.far) hipLaunchKernelGGL((attn_bwd_dkdv_kernel<T, D, false, true, false>), grid, block, 0, stream, a);
+        else hipLaunchKernelGGL((attn_bwd_dkdv_kernel<T, D, false, false, false>), grid, block, 0, stream, a);
       }
       int rc = check_launch("attn_bwd dkdv");
       if (rc != RSWA_OK) return rc;
@@ -1217,7 +1554,25 @@ int launch_bwd(AttnArgs& a, hipStream_t stream, int phases) {
       if (rc != RSWA_OK) return rc;
     }
   }
-  if (phases & RSWA_BWD_DQ) {
+  if ((phases & RSWA_BWD_DQ) && a.ds) {
+    const int hsh = (a.group & 3) == 0 ? 2 : (a.group & 1) == 0 ? 1 : 0;
+    const int bm = 256 >> hsh;
+    const int units_q = (a.group >> hsh) * a.heads_kv;
+    if (a.cu_q) {
+      a.n_tile = (int)(ceil_div(a.rows_q, bm) + a.batch);
+      a.n_work = a.n_tile * units_q;
+    } else {
+      a.n_tile = (int)ceil_div(a.seqlen_q, bm);
+      a.n_work = a.n_tile * units_q * a.batch;
+    }
+    if (a.n_work > 0) {
+      clear_launch_error();
+      hipLaunchKernelGGL((attn_bwd_dq_ds_kernel<T, D>), dim3(padded_grid(a.n_work)), dim3(256), 0,
+                         stream, a);
+      int rc = check_launch("attn_bwd dq (dS hand-off)");
+      if (rc != RSWA_OK) return rc;
+    }
+  } else if (phases & RSWA_BWD_DQ) {
     const bool pair = (a.group & 1) == 0;
     const bool small = a.avg_keys <= RSWA_DQ_SMALL_AVG_KEYS;
     const int bm = (pair ? 16 : 32) * (small ? 4 : 8);
@@ -1251,9 +1606,10 @@ int launch_bwd(AttnArgs& a, hipStream_t stream, int phases) {
 
 namespace rswa {
 namespace {
-int bwd_entry(const rswa_attn_params* p, void* stream, int phases, bool allow_split) {
+int bwd_entry(const rswa_attn_params* p, void* stream, int phases, bool allow_split,
+              bool allow_handoff) {
   AttnArgs a;
-  int rc = fill_args(p, true, a, allow_split);
+  int rc = fill_args(p, true, a, allow_split, allow_handoff);
   if (rc != RSWA_OK) return rc;
   hipStream_t st = (hipStream_t)stream;
   if (p->dtype == RSWA_BF16) {
@@ -1267,7 +1623,7 @@ int bwd_entry(const rswa_attn_params* p, void* stream, int phases, bool allow_sp
 }  // namespace rswa
 
 extern "C" int rswa_attn_bwd_phases(const rswa_attn_params* p, void* stream, int phases) {
-  return rswa::bwd_entry(p, stream, phases, true);
+  return rswa::bwd_entry(p, stream, phases, true, true);
 }
 
 extern "C" int rswa_attn_bwd(const rswa_attn_params* p, void* stream) {
@@ -1331,5 +1687,5 @@ extern "C" int rswa_attn_bwd_static(const rswa_attn_params* p, void* stream) {
   void* ptr = scratch_on_current_device();
   if (!ptr) return RSWA_ERR_LAUNCH;
   q.workspace = ptr;
-  return bwd_entry(&q, stream, RSWA_BWD_PREP | RSWA_BWD_DKDV | RSWA_BWD_DQ, false);
+  return bwd_entry(&q, stream, RSWA_BWD_PREP | RSWA_BWD_DKDV | RSWA_BWD_DQ, false, false);
 }

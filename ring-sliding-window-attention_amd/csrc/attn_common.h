@@ -72,6 +72,14 @@ struct AttnArgs {
   int32_t seg;
   int32_t avg_keys;  // keys a query row sees on average (host estimate; block shapes hang on it)
   int32_t far;  // a sequence of some streamed tensor spans 2 GiB or more: FAR kernels
+  // dS hand-off (backward): the dK/dV kernel stores its packed 16-bit dS tiles and the dQ
+  // kernel of that route only multiplies them with K.  Unit = 32 query rows x 64 keys (one
+  // wave's step), 4 KiB, at ds + (((q head * ds_slots + row-tile slot) * ds_nkb + key block %
+  // ds_nkb) * 4 + 64-key group) * 4096; a row tile sees at most ds_nkb consecutive 256-key
+  // blocks.  Null: the dQ kernel recomputes S and dP.
+  char* ds;
+  int32_t ds_nkb;
+  int32_t ds_slots;  // 32-row tile slots per q head (dense: batch * tiles; packed: rows / 32 + batch)
   float scale, scale_log2;
 };
 
@@ -408,6 +416,16 @@ __device__ __forceinline__ void lds_barrier() {
   asm volatile("" ::: "memory");
 }
 __device__ __forceinline__ void wait_dma() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+// Wait until at most N of this wave's vector memory operations (loads, loads into LDS, stores:
+// they complete in issue order) are outstanding.  Through the builtin, so that the compiler's own
+// bookkeeping of what is in flight sees the wait (gfx9 encoding: vmcnt in bits 3:0 and 15:14,
+// the other counters left at their "no wait" values).
+template <int N>
+__device__ __forceinline__ void wait_vmem_but() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+  asm volatile("" ::: "memory");
+}
 
 // max / sum across the two half-waves (lane l <-> lane l ^ 32).
 __device__ __forceinline__ float halfwave_max(float x) {
@@ -429,6 +447,10 @@ __device__ __forceinline__ float halfwave_sum(float x) {
 // prologue, partial store and share of the final sum -- so launches that already give every
 // compute unit a block are left alone.
 constexpr int kDkvKeysPerBlock = 256;
+// dS hand-off: bytes one dK/dV block leaves per 32-row query tile (32 x 256 16-bit values) and
+// per wave of it (32 x 64: the unit the dQ kernel of that route fetches)
+constexpr int kDsBlockBytes = 32 * kDkvKeysPerBlock * 2;
+constexpr int kDsUnitBytes = kDsBlockBytes / 4;
 constexpr int kMaxTileRows = 256;  // bound on the rows fetched as one tile that the stride checks assume
                                    // (today's largest tile has 64 rows: K / V in the forward and dQ kernels)
 constexpr int kComputeUnits = 256;  // MI355X
@@ -445,12 +467,16 @@ struct BwdLayout {
   int sink_chunks;         // row chunks of the sink kernel per (sequence, kv head); 0: no sink kernel
   int sink_count_index;    // its first arrival counter
   uint64_t sink_off;       // its fp32 sums
+  // dS hand-off (ds_bytes == 0: not used for this call)
+  uint64_t ds_off, ds_bytes;
+  int ds_nkb, ds_slots;
 };
-BwdLayout bwd_layout(const rswa_attn_params* p, bool allow_split);
+BwdLayout bwd_layout(const rswa_attn_params* p, bool allow_split, bool allow_handoff = false);
 
 // Fill an AttnArgs from the public struct; validates what both directions share.
 // `allow_split` = false keeps the dK/dV kernel at one block per key tile, whatever the shape
 // (workspace holds the statistics only).
-int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a, bool allow_split = true);
+int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a, bool allow_split = true,
+              bool allow_handoff = false);
 
 }  // namespace rswa

@@ -78,6 +78,7 @@ class AttnParams(Structure):
         ("v2", c_void_p),
         ("dk2", c_void_p),
         ("dv2", c_void_p),
+        ("ds_handoff", c_int32),
     ]
 
 
@@ -125,6 +126,8 @@ def load(path: str) -> ctypes.CDLL:
     L.rswa_attn_bwd_phases.argtypes = [POINTER(AttnParams), c_void_p, c_int]
     L.rswa_attn_bwd_workspace_bytes.restype = c_uint64
     L.rswa_attn_bwd_workspace_bytes.argtypes = [POINTER(AttnParams)]
+    L.rswa_attn_bwd_handoff_active.restype = c_int
+    L.rswa_attn_bwd_handoff_active.argtypes = [POINTER(AttnParams)]
     if L.rswa_sizeof_attn_params() != ctypes.sizeof(AttnParams):
         raise ImportError(
             "rswa_attn_params layout mismatch between librswa.so "

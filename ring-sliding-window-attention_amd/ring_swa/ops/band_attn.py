@@ -204,6 +204,7 @@ def attn_bwd(
     dq_accumulate: bool = False,
     static_workspace: bool = False,
     second: Optional[Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]] = None,
+    handoff=None,
 ) -> None:
     """Masked attention backward; overwrites ``dq, dk, dv`` (views are fine).
 
@@ -217,7 +218,18 @@ def attn_bwd(
     already in ``dq`` (fp32 add of the two 16-bit values, one rounding).
     ``static_workspace=True`` runs the whole backward on the library's built-in statistics
     buffer (``rswa_attn_bwd_static``): no device memory is allocated by the call; sizes
-    beyond the buffer raise ``NotImplementedError`` and overlapping calls on one GPU race."""
+    beyond the buffer raise ``NotImplementedError`` and overlapping calls on one GPU race.
+
+    ``handoff``: dS hand-off (``ds_handoff`` of the ABI) -- the dK/dV kernel stores its 16-bit dS
+    tiles in the workspace and dQ comes from a kernel that only multiplies them with K instead
+    of recomputing S and dP.  ``None`` (default) takes it when the library accepts the shape and
+    the tiles fit ``handoff_max_bytes()`` (0 unless the environment switches the route on: it is
+    not faster at the sizes measured); ``True`` asks for it whatever its size (shapes the
+    library does not accept still take the recomputing route, and so do small launches whose key
+    tiles the dK/dV kernel splits over several blocks -- ``"force"`` prefers the hand-off to that
+    split); ``False`` never.  With
+    ``phases`` spread over several calls the same value must be passed to each, on the same
+    workspace, and the dK/dV phase must run before the dQ phase."""
     packed = cu_seqlens_q is not None
     _check_qkv(q, k, v, packed)
     assert second is None or k.numel() > 0, "two key ranges: the first must not be empty"
@@ -273,6 +285,7 @@ def attn_bwd(
         with torch.cuda.device(dev):
             _lib.check(L.rswa_attn_bwd_static(p, _lib.stream_ptr(dev)))
         return
+    _set_handoff(p, handoff)
     need = int(L.rswa_attn_bwd_workspace_bytes(p))
     if workspace is None:
         workspace = torch.empty(need, dtype=torch.uint8, device=dev)  # 512-B aligned by torch
@@ -283,17 +296,69 @@ def attn_bwd(
         _lib.check(L.rswa_attn_bwd_phases(p, _lib.stream_ptr(dev), int(phases)))
 
 
+def handoff_max_bytes() -> int:
+    """Largest dS buffer ``attn_bwd(handoff=None)`` takes by itself.  0 unless the environment
+    asks for the route (``RSWA_DS_HANDOFF=1``; then ``RSWA_DS_HANDOFF_MAX_BYTES`` or 8 GiB): measured
+    on an MI355X the route is within +-5 % of the recomputing one at every size tried (faster
+    at windows of a few hundred keys, slower at thousands: writing and reading 2 bytes per
+    (query, key) pair costs what the saved matrix work gains), so it is not taken by default."""
+    if os.environ.get("RSWA_DS_HANDOFF", "0") != "1":
+        return 0
+    return int(os.environ.get("RSWA_DS_HANDOFF_MAX_BYTES", 8 << 30))
+
+
+def _set_handoff(p, handoff: Optional[bool]) -> bool:
+    """Decide ``p.ds_handoff`` (see ``attn_bwd``); returns whether the library will take it."""
+    L = _lib.lib()
+    p.ds_handoff = 0
+    if handoff is False:
+        return False
+    p.ds_handoff = 2 if handoff == "force" else 1
+    if not L.rswa_attn_bwd_handoff_active(p):
+        p.ds_handoff = 0
+        return False
+    if handoff is None:
+        if handoff_max_bytes() == 0:
+            p.ds_handoff = 0
+            return False
+        with_ds = int(L.rswa_attn_bwd_workspace_bytes(p))
+        p.ds_handoff = 0
+        if with_ds - int(L.rswa_attn_bwd_workspace_bytes(p)) > handoff_max_bytes():
+            return False
+        p.ds_handoff = 1
+    return True
+
+
 def bwd_workspace_bytes(q: torch.Tensor, k: torch.Tensor,
                         cu_seqlens_q: Optional[torch.Tensor] = None,
                         cu_seqlens_k: Optional[torch.Tensor] = None, *,
-                        second_rows: int = 0) -> int:
+                        second_rows: int = 0,
+                        window_size: Tuple[int, int] = (-1, -1), causal: bool = False,
+                        num_sink: int = 0, handoff: Optional[bool] = False) -> int:
     """Scratch size of one backward over ``q`` against ``k`` (dense ``[B,S,H,D]`` or packed
     ``[T,H,D]``), as ``rswa_attn_bwd_workspace_bytes`` computes it: two fp32 values per
-    (row, q head), plus the partial sums of the dK/dV kernel when the shape makes it deal the
-    q heads of a GQA group to several blocks."""
-    p = _params(q, k, k, 1.0, (-1, -1), False, cu_seqlens_q, cu_seqlens_k, 0)
+    (row, q head); the partial sums of the dK/dV kernel when the shape makes it deal the q
+    heads of a GQA group to several blocks; the sums of the sink kernel with ``num_sink`` keys
+    under a bounded window; the dS tiles with ``handoff`` (which depend on the window).  Pass the
+    mask and ``handoff`` of the ``attn_bwd`` call the workspace is for."""
+    p = _params(q, k, k, 1.0, window_size, causal, cu_seqlens_q, cu_seqlens_k, num_sink)
     p.seqlen_k += int(second_rows)  # keys in two row ranges: the rows of the second
+    p.dout_stride = p.q_stride
+    _set_handoff(p, handoff)
     return int(_lib.lib().rswa_attn_bwd_workspace_bytes(p))
+
+
+def bwd_handoff_active(q: torch.Tensor, k: torch.Tensor,
+                       cu_seqlens_q: Optional[torch.Tensor] = None,
+                       cu_seqlens_k: Optional[torch.Tensor] = None, *,
+                       second_rows: int = 0,
+                       window_size: Tuple[int, int] = (-1, -1), causal: bool = False,
+                       num_sink: int = 0, handoff: Optional[bool] = None) -> bool:
+    """Would ``attn_bwd`` with these arguments take the dS hand-off route?"""
+    p = _params(q, k, k, 1.0, window_size, causal, cu_seqlens_q, cu_seqlens_k, num_sink)
+    p.seqlen_k += int(second_rows)
+    p.dout_stride = p.q_stride
+    return _set_handoff(p, handoff)
 
 
 # ---- names of the upstream wrappers -----------------------------------------
