@@ -367,15 +367,12 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": "c3_rank_share",
-            "detail": "1 rank of virtual cp 8: chunk 8192 of seq 65536, 32 q / 8 kv heads, "
-                      "head_dim 128, window 4096; fwd+bwd via autograd; ring_dtypes=False: the window "
-                      "is shorter than the chunk, so the rank's keys -- the previous chunk's last "
-                      "4096 rows, then its own chunk, each taken where it lies -- are one band pass "
-                      "(one forward, one dK/dV and one dQ launch; the same sums as the reference's "
-                      "own-chunk block + previous-chunk corner block + LSE merge, without the rounding "
-                      "of a partial output).  That two-block form with the reference's accumulator "
-                      "types (fp32 output, fp64 LSE, one merge per block) is ring_dtypes=True, timed "
-                      "as ms_per_step_ring_dtypes",
+            "detail": "1 rank of virtual cp 8: chunk 8192 of seq 65536, 32 q / 8 kv heads, head_dim "
+                      "128, window 4096; fwd+bwd via autograd; route one_pass: the previous chunk's "
+                      "last 4096 rows and the own chunk, each where it lies, as one band pass "
+                      "(ms_per_step_two_blocks / ms_per_step_ring_dtypes: the reference's two blocks + "
+                      "LSE merge, with 16-bit and with fp32 / fp64 accumulators)",
+            "route": "one_pass",
             "ring_dtypes": False,
             "batch": 1, "chunk": S, "heads_q": HQ, "heads_kv": HK, "head_dim": D, "window": W,
             "pairs_per_head": pairs, "flops_per_step": flops,
@@ -390,14 +387,24 @@ def main():
         out = ring_swa.ring_rank_share_attn(q, k, v, [prev], W, CP, RANK, ring_dtypes=True)
         out.backward(do)
 
-    for _ in range(3):
-        step_ring_dtypes()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step_ring_dtypes()
-    torch.cuda.synchronize()
-    rec["ms_per_step_ring_dtypes"] = (time.perf_counter() - t0) * 1e3 / args.steps
+    # ... and as the reference's two blocks merged in 16 bits (own-chunk block, previous-chunk
+    # corner block merged in the second forward's epilogue, dq summed in the own-chunk dQ kernel)
+    def step_two_blocks():
+        for t in (q, k, v, prev):
+            t.grad = None
+        out = ring_swa.ring_rank_share_attn(q, k, v, [prev], W, CP, RANK, one_pass=False)
+        out.backward(do)
+
+    for name, fn in (("ms_per_step_ring_dtypes", step_ring_dtypes),
+                     ("ms_per_step_two_blocks", step_two_blocks)):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            fn()
+        torch.cuda.synchronize()
+        rec[name] = (time.perf_counter() - t0) * 1e3 / args.steps
 
     # ---- roofline of the dominant kernel: the backward dK/dV kernel on the step's band ----
     # (8192 queries against the previous chunk's 4096-row tail and the own chunk, window 4096:
@@ -521,6 +528,20 @@ def main():
                     c5[f"{impl}_sinks{n_sink}"] = rate(info5["pairs"], t5)
                     del c5_step
             rec["c5_slm_varlen_t65536_w4092"] = c5
+            # a pack of 4096 sequences of 16 tokens (8 q / 2 kv heads, window 8): every block has
+            # to find its sequence among 4096 -- a linear search took milliseconds here
+            n_seq, L_seq = 4096, 16
+            cu_m = torch.arange(0, (n_seq + 1) * L_seq, L_seq, dtype=torch.int32, device=dev)
+            qm, dom = mk(n_seq * L_seq, 8, D), mk(n_seq * L_seq, 8, D)
+            km, vm = mk(n_seq * L_seq, 2, D), mk(n_seq * L_seq, 2, D)
+            gm = [torch.empty_like(t) for t in (qm, km, vm)]
+
+            def many():
+                om, lm = attn_fwd(qm, km, vm, None, (8, 0), True, cu_m, cu_m)
+                attn_bwd(qm, km, vm, om, lm, dom, *gm, None, (8, 0), True, cu_m, cu_m)
+
+            rec["pack_of_4096_sequences_of_16_fwd_bwd_ms"] = event_ms(many, 10)[0]
+            del qm, dom, km, vm, gm
             T5 = 65536
             # the merge of that configuration's split path: all tokens x 32 heads, 16-bit
             # outputs and fp32 LSE on both sides (780 bytes per row)
@@ -547,6 +568,18 @@ def main():
                                 "GB/s": nbytes / med / 1e6,
                                 "dtypes": "o fp32, new o bf16, lse fp64, new lse fp32"}
                 if name == "sweep_s131072":
+                    # the same number of bytes through the library's plain copy kernel (half
+                    # read, half written), same run: what a kernel that only moves memory reaches
+                    from ring_swa.ops.lse_merge import stream_copy
+
+                    src = torch.empty(nbytes // 2 // 16 * 16, dtype=torch.uint8, device=dev)
+                    dst = torch.empty_like(src)
+                    cmed, cavg = event_ms(lambda: stream_copy(dst, src), 20)
+                    rec["copy_GBps"] = 2 * src.numel() / cavg / 1e6
+                    merges["sweep_s131072"]["copy_kernel_same_bytes"] = {
+                        "us": cavg * 1e3, "GB/s": rec["copy_GBps"],
+                        "merge_over_copy": (nbytes / avg) / (2 * src.numel() / cavg)}
+                    del src, dst
                     rec["roofline_merge"] = {
                         "kernel": "merge_kernel<float,bf16,16>", "bound": "hbm",
                         "achieved": nbytes / avg / 1e6, "peak": PEAK_HBM_GBPS, "unit": "GB/s",

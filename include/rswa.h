@@ -75,6 +75,16 @@ int rswa_merge_attn_out(void* o, int o_dtype, const int64_t* o_stride,
                         void* stream);
 
 /*
+ * Plain device-to-device copy of `bytes` bytes (a multiple of 16; both pointers 16-byte
+ * aligned, ranges not overlapping) by a kernel that does nothing else: 16 bytes a lane,
+ * non-temporal.  No counterpart in the upstream package, whose merge harness
+ * (ring_swa/ops/merge.py:257-302) only times the merge: this is the yardstick beside it -- the
+ * rate a kernel that only moves memory reaches on the same device in the same run -- against
+ * which rswa_merge_attn_out's rate is reported.
+ */
+int rswa_stream_copy(void* dst, const void* src, uint64_t bytes, void* stream);
+
+/*
  * One attention block, forward or backward.
  *
  * Dense mode (cu_seqlens_q == NULL): q/out/dout/dq are [batch, seqlen_q,
@@ -240,6 +250,15 @@ int rswa_attn_bwd_phases(const rswa_attn_params* p, void* stream, int phases);
  */
 #define RSWA_BWD_STATIC_MAX_BYTES (32u << 20)
 int rswa_attn_bwd_static(const rswa_attn_params* p, void* stream);
+
+/* Looks up the address of that buffer on the current device, which the first
+ * rswa_attn_bwd_static call on a device otherwise does itself (a symbol look-up that may load
+ * the library's device image, under a host mutex).  A caller that captures rswa_attn_bwd_static
+ * into a HIP graph calls this once per device BEFORE the capture begins: the look-up is no
+ * stream operation and must not happen inside a capture.  Launches nothing, allocates nothing;
+ * calling it again is free.  No counterpart in the upstream package (it serves the same callers
+ * as rswa_attn_bwd_static: those that cannot allocate). */
+int rswa_attn_bwd_static_init(void);
 
 /* Scratch rswa_attn_bwd needs for these shapes: two fp32 values per (row, q head) -- the
  * row sum of dout * out and the LSE in base-2 units -- and, for launches with so few key

@@ -1665,6 +1665,10 @@ void* scratch_on_current_device() {
 }  // namespace
 }  // namespace rswa
 
+extern "C" int rswa_attn_bwd_static_init(void) {
+  return rswa::scratch_on_current_device() ? RSWA_OK : RSWA_ERR_LAUNCH;
+}
+
 extern "C" int rswa_attn_bwd_static(const rswa_attn_params* p, void* stream) {
   using namespace rswa;
   RSWA_REQUIRE(p != nullptr, RSWA_ERR_INVALID, "attn_bwd_static: null params");

@@ -9,6 +9,8 @@
 // accesses; all loads of a thread's rows are issued before the first use.
 #include "rswa_common.h"
 
+#include <type_traits>
+
 namespace rswa {
 namespace {
 
@@ -153,8 +155,107 @@ __global__ __launch_bounds__(kThreads) void merge_kernel(const MergeArgs a) {
   }
 }
 
+#ifdef RSWA_MERGE_E4
+// experiment: 4 elements per lane (every wave instruction fully coalesced), ROWS rows per thread
+template <typename T> struct Vec4;
+template <> struct Vec4<float> {
+  static __device__ __forceinline__ void load(const float* p, float (&x)[4]) {
+    f32x4 a = __builtin_nontemporal_load((const f32x4*)p);
+    for (int i = 0; i < 4; i++) x[i] = a[i];
+  }
+  static __device__ __forceinline__ void store(float* p, const float (&x)[4]) {
+    f32x4 a = {x[0], x[1], x[2], x[3]};
+    __builtin_nontemporal_store(a, (f32x4*)p);
+  }
+};
+template <> struct Vec4<__bf16> {
+  static __device__ __forceinline__ void load(const __bf16* p, float (&x)[4]) {
+    u32x2 a = __builtin_nontemporal_load((const u32x2*)p);
+    for (int i = 0; i < 2; i++) {
+      x[2 * i] = __uint_as_float(a[i] << 16);
+      x[2 * i + 1] = __uint_as_float(a[i] & 0xffff0000u);
+    }
+  }
+  static __device__ __forceinline__ void store(__bf16* p, const float (&x)[4]) {
+    f32x4 f = {x[0], x[1], x[2], x[3]};
+    bf16x4 h = __builtin_convertvector(f, bf16x4);
+    __builtin_nontemporal_store(h, (bf16x4*)p);
+  }
+};
+#ifndef RSWA_MERGE_E4_ROWS
+#define RSWA_MERGE_E4_ROWS 8
+#endif
+template <typename TO, typename TN>
+__global__ __launch_bounds__(kThreads) void merge_kernel_e4(const MergeArgs a) {
+  constexpr int LPR = 32, RP = kThreads / LPR, NR = RSWA_MERGE_E4_ROWS, BS = RP * NR;
+  const int bid = blockIdx.x;
+  const int h = bid % a.heads;
+  const int rest = bid / a.heads;
+  const int st = rest % a.n_stile;
+  const int b = rest / a.n_stile;
+  const int r = threadIdx.x / LPR;
+  const int c = (threadIdx.x % LPR) * 4;
+  TO* o = (TO*)a.o + (int64_t)b * a.o_st[0] + (int64_t)h * a.o_st[2] + c;
+  const TN* on = (const TN*)a.on + (int64_t)b * a.on_st[0] + (int64_t)h * a.on_st[2] + c;
+  const int64_t l_base = (int64_t)b * a.l_st[0] + (int64_t)h * a.l_st[1];
+  const int64_t ln_base = (int64_t)b * a.ln_st[0] + (int64_t)h * a.ln_st[1];
+  float xo[NR][4], xn[NR][4], la[NR], lb[NR];
+  const int s0 = st * BS + r;
+#pragma unroll
+  for (int i = 0; i < NR; i++) {
+    const int s = s0 + i * RP;
+    if (s < a.seqlen) {
+      la[i] = a.lse_f64 ? (float)((const double*)a.lse)[l_base + (int64_t)s * a.l_st[2]]
+                        : ((const float*)a.lse)[l_base + (int64_t)s * a.l_st[2]];
+      lb[i] = a.lsen_f64 ? (float)((const double*)a.lsen)[ln_base + (int64_t)s * a.ln_st[2]]
+                         : ((const float*)a.lsen)[ln_base + (int64_t)s * a.ln_st[2]];
+      Vec4<TO>::load(o + (int64_t)s * a.o_st[1], xo[i]);
+      Vec4<TN>::load(on + (int64_t)s * a.on_st[1], xn[i]);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < NR; i++) {
+    const int s = s0 + i * RP;
+    if (s < a.seqlen) {
+      const float ninf = -__builtin_inff();
+      const bool both_empty = (la[i] == ninf) && (lb[i] == ninf);
+      const float diff = both_empty ? 0.f : lb[i] - la[i];
+      const float w_old = both_empty ? 0.f : 1.f / (1.f + __expf(diff));
+      const float w_new = both_empty ? 0.f : 1.f / (1.f + __expf(-diff));
+      float y[4];
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const float t0 = (w_old == 0.f) ? 0.f : xo[i][j] * w_old;
+        const float t1 = (w_new == 0.f) ? 0.f : xn[i][j] * w_new;
+        y[j] = t0 + t1;
+      }
+      Vec4<TO>::store(o + (int64_t)s * a.o_st[1], y);
+      if ((threadIdx.x % LPR) == 0) {
+        const float m = fmaxf(la[i], lb[i]);
+        const float merged = both_empty ? ninf : m + log1pf(__expf(-fabsf(diff)));
+        if (a.lse_f64) ((double*)a.lse)[l_base + (int64_t)s * a.l_st[2]] = (double)merged;
+        else ((float*)a.lse)[l_base + (int64_t)s * a.l_st[2]] = merged;
+      }
+    }
+  }
+}
+#endif
+
 template <typename TO, typename TN>
 int launch_merge(const MergeArgs& a, int64_t batch, hipStream_t stream) {
+#ifdef RSWA_MERGE_E4
+  if constexpr ((std::is_same_v<TO, float> || std::is_same_v<TO, __bf16>) && std::is_same_v<TN, __bf16>) {
+    if (a.head_dim == 128) {
+      MergeArgs args = a;
+      constexpr int BS = (kThreads / 32) * RSWA_MERGE_E4_ROWS;
+      args.n_stile = (int)ceil_div(a.seqlen, BS);
+      const int64_t blocks = (int64_t)args.n_stile * a.heads * batch;
+      clear_launch_error();
+      hipLaunchKernelGGL((merge_kernel_e4<TO, TN>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, args);
+      return check_launch("merge_attn_out");
+    }
+  }
+#endif
   const int chunks = (a.head_dim + 7) / 8;
   int lpr = 1;
   while (lpr < chunks) lpr *= 2;
@@ -180,6 +281,22 @@ int launch_merge(const MergeArgs& a, int64_t batch, hipStream_t stream) {
   return check_launch("merge_attn_out");
 }
 
+// Plain streaming copy, 16 bytes a lane, four loads of a thread in flight before its first
+// store, non-temporal both ways: the yardstick for what a kernel that only moves memory reaches
+// on the device it runs on.
+__global__ __launch_bounds__(kThreads) void stream_copy_kernel(u32x4* __restrict__ dst,
+                                                               const u32x4* __restrict__ src,
+                                                               int64_t n16) {
+  const int64_t base = (int64_t)blockIdx.x * (kThreads * 4) + threadIdx.x;
+  u32x4 v[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+    if (base + i * kThreads < n16) v[i] = __builtin_nontemporal_load(src + base + i * kThreads);
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+    if (base + i * kThreads < n16) __builtin_nontemporal_store(v[i], dst + base + i * kThreads);
+}
+
 int elem_bytes(int dt) {
   switch (dt) {
     case RSWA_BF16:
@@ -192,6 +309,21 @@ int elem_bytes(int dt) {
 
 }  // namespace
 }  // namespace rswa
+
+extern "C" int rswa_stream_copy(void* dst, const void* src, uint64_t bytes, void* stream) {
+  using namespace rswa;
+  RSWA_REQUIRE(dst && src, RSWA_ERR_INVALID, "stream_copy: null pointer");
+  RSWA_REQUIRE(((uintptr_t)dst) % 16 == 0 && ((uintptr_t)src) % 16 == 0 && bytes % 16 == 0,
+               RSWA_ERR_UNSUPPORTED, "stream_copy: pointers and size must be multiples of 16 bytes");
+  const int64_t n16 = (int64_t)(bytes / 16);
+  const int64_t blocks = ceil_div(n16, kThreads * 4);
+  RSWA_REQUIRE(blocks < (1ll << 31), RSWA_ERR_UNSUPPORTED, "stream_copy: more than 32 TiB");
+  if (blocks == 0) return RSWA_OK;
+  clear_launch_error();
+  hipLaunchKernelGGL(stream_copy_kernel, dim3((unsigned)blocks), dim3(kThreads), 0,
+                     (hipStream_t)stream, (u32x4*)dst, (const u32x4*)src, n16);
+  return check_launch("stream_copy");
+}
 
 extern "C" int rswa_merge_attn_out(void* o, int o_dtype, const int64_t* o_stride, void* lse,
                                    int lse_dtype, const int64_t* lse_stride, const void* o_new,

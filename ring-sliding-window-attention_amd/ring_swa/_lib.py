@@ -118,10 +118,14 @@ def load(path: str) -> ctypes.CDLL:
         c_void_p, c_int, POINTER(c_int64),
         c_int64, c_int64, c_int64, c_int64, c_void_p,
     ]
+    L.rswa_stream_copy.restype = c_int
+    L.rswa_stream_copy.argtypes = [c_void_p, c_void_p, c_uint64, c_void_p]
     for name in ("rswa_attn_fwd", "rswa_attn_bwd", "rswa_attn_bwd_static"):
         fn = getattr(L, name)
         fn.restype = c_int
         fn.argtypes = [POINTER(AttnParams), c_void_p]
+    L.rswa_attn_bwd_static_init.restype = c_int
+    L.rswa_attn_bwd_static_init.argtypes = []
     L.rswa_attn_bwd_phases.restype = c_int
     L.rswa_attn_bwd_phases.argtypes = [POINTER(AttnParams), c_void_p, c_int]
     L.rswa_attn_bwd_workspace_bytes.restype = c_uint64

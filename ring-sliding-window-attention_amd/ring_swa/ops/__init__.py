@@ -15,7 +15,13 @@ from .band_attn import (
     wrapped_flash_attn_fwd_varlen,
 )
 from .lse_merge import merge_attn_out
-from .p2p import get_group_local_to_global_rank_map, ring_attn_p2p_communicate
+from .p2p import (
+    broadcast_tensor_to_group,
+    exchange_and_sum_tensors,
+    get_group_local_to_global_rank_map,
+    reduce_sum_tesnsor_to_rank,
+    ring_attn_p2p_communicate,
+)
 
 __all__ = [
     "attn_fwd",
@@ -30,5 +36,8 @@ __all__ = [
     "flash_attn_varlen_bwd_func",
     "merge_attn_out",
     "ring_attn_p2p_communicate",
+    "broadcast_tensor_to_group",
+    "reduce_sum_tesnsor_to_rank",
+    "exchange_and_sum_tensors",
     "get_group_local_to_global_rank_map",
 ]

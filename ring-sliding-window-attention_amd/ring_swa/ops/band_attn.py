@@ -296,6 +296,14 @@ def attn_bwd(
         _lib.check(L.rswa_attn_bwd_phases(p, _lib.stream_ptr(dev), int(phases)))
 
 
+def bwd_static_init(device=None) -> None:
+    """Resolve the address of the built-in statistics buffer of ``attn_bwd(static_workspace=True)``
+    on ``device`` (default: the current one).  The first such backward on a device does it by
+    itself; call this before capturing one into a HIP graph, where the look-up must not happen."""
+    with torch.cuda.device(device):
+        _lib.check(_lib.lib().rswa_attn_bwd_static_init())
+
+
 def handoff_max_bytes() -> int:
     """Largest dS buffer ``attn_bwd(handoff=None)`` takes by itself.  0 unless the environment
     asks for the route (``RSWA_DS_HANDOFF=1``; then ``RSWA_DS_HANDOFF_MAX_BYTES`` or 8 GiB): measured

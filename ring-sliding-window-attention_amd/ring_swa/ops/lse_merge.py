@@ -40,3 +40,16 @@ def merge_attn_out(
             b, s, h, d, _lib.stream_ptr(dev),
         )
     _lib.check(st)
+
+
+def stream_copy(dst: torch.Tensor, src: torch.Tensor) -> None:
+    """``dst <- src`` (contiguous device tensors of the same byte size, a multiple of 16) with
+    the library's plain streaming-copy kernel: the yardstick the benchmark reports beside the
+    merge kernel's rate (what a kernel that only moves memory reaches on the same device)."""
+    assert dst.is_contiguous() and src.is_contiguous()
+    nbytes = src.numel() * src.element_size()
+    assert nbytes == dst.numel() * dst.element_size() and nbytes % 16 == 0
+    dev = _lib.require_device(dst, src)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().rswa_stream_copy(dst.data_ptr(), src.data_ptr(), nbytes,
+                                               _lib.stream_ptr(dev)))

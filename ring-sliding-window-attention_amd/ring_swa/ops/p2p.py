@@ -1,8 +1,11 @@
 """Point-to-point exchange of KV / dKV chunks between context-parallel ranks, and the
 group-local -> global rank map.
 
-Takes the place of ``ring_swa/ops/comm.py:8-40`` (``ring_attn_p2p_communicate``) and
-``:152-232`` (``get_group_local_to_global_rank_map``) of the upstream package.  Works on any
+Takes the place of ``ring_swa/ops/comm.py:8-40`` (``ring_attn_p2p_communicate``),
+``:43-149`` (``broadcast_tensor_to_group``, ``reduce_sum_tesnsor_to_rank``,
+``exchange_and_sum_tensors``: the helpers of upstream's streaming-LLM ring, kept under their
+names -- the ring of this package moves its sink rows point to point and does not call them)
+and ``:152-232`` (``get_group_local_to_global_rank_map``) of the upstream package.  Works on any
 ``torch.distributed`` backend: ``"nccl"`` (RCCL over xGMI on MI355X nodes) with device
 tensors, ``"gloo"`` with host tensors (the CPU test tier of the ring logic).
 
@@ -73,3 +76,82 @@ def ring_attn_p2p_communicate(rank: int, send_tensor: torch.Tensor, send_rank: i
     (``ops/comm.py:8-40``; ``rank`` ordered its sends and receives by parity to avoid a
     deadlock, which the batched form does not need)."""
     return exchange([(send_tensor, send_rank)], [(recv_tensor, recv_rank)], cp_group)
+
+
+class _StagedCollective:
+    """Work handle of a collective on a gloo group whose tensor lives on a device: the data
+    travelled in a host copy, ``wait`` completes the collective and, where the rank receives,
+    copies the result back."""
+
+    def __init__(self, work, tensor, host, receives):
+        self._work, self._tensor, self._host, self._receives = work, tensor, host, receives
+
+    def wait(self):
+        self._work.wait()
+        if self._receives and self._host is not None:
+            self._tensor.copy_(self._host)
+            self._host = None
+        return True
+
+
+def _staged(tensor: torch.Tensor, group):
+    """``(tensor the collective runs on, needs copy-back)``: gloo takes host tensors only."""
+    if tensor.is_cuda and dist.get_backend(group) == "gloo":
+        return tensor.cpu(), True
+    return tensor, False
+
+
+def broadcast_tensor_to_group(tensor: torch.Tensor, src_rank: int, cp_group):
+    """Asynchronous broadcast of ``tensor`` from global rank ``src_rank`` to every rank of
+    ``cp_group`` (``ops/comm.py:43-70``): returns a handle whose ``wait()`` completes it.
+    Every rank of the group calls it with a tensor of the same shape and dtype."""
+    host, staged = _staged(tensor, cp_group)
+    work = dist.broadcast(host, src=src_rank, group=cp_group, async_op=True)
+    if not staged:
+        return work
+    return _StagedCollective(work, tensor, host, dist.get_rank() != src_rank)
+
+
+def reduce_sum_tesnsor_to_rank(tensor: torch.Tensor, dst_rank: int, cp_group) -> torch.Tensor:
+    """Sum of every rank's ``tensor`` on global rank ``dst_rank``, in place (``ops/comm.py:73-100``,
+    upstream's spelling of the name); blocking; returns ``tensor`` (on the other ranks its
+    contents are unspecified afterwards, as with ``dist.reduce``)."""
+    host, staged = _staged(tensor, cp_group)
+    dist.reduce(host, dst=dst_rank, op=dist.ReduceOp.SUM, group=cp_group)
+    if staged and dist.get_rank() == dst_rank:
+        tensor.copy_(host)
+    return tensor
+
+
+def exchange_and_sum_tensors(tensor_to_send: torch.Tensor, send_to_rank: int, cp_group) -> torch.Tensor:
+    """Every rank sends its tensor to ONE rank of its choice (group-local index
+    ``send_to_rank``, as upstream's all-to-all slot, ``ops/comm.py:103-149``); returns the sum of
+    what this rank received (zeros if nobody sent to it).  Blocking; same shape and dtype on
+    every rank.
+
+    Upstream fills an all-to-all with a zero tensor for every rank that is not the destination
+    (world size times the payload in flight).  Here the ranks first share their destinations (one
+    integer each), then only the real payloads travel, point to point; they are added in rank
+    order, so the sum does not depend on arrival order."""
+    world = dist.get_world_size(group=cp_group)
+    me = dist.get_rank(group=cp_group)
+    members = dist.get_process_group_ranks(cp_group)
+    dests = [torch.zeros(1, dtype=torch.int64) for _ in range(world)]
+    mine = torch.tensor([int(send_to_rank)], dtype=torch.int64)
+    if dist.get_backend(cp_group) != "gloo":
+        mine = mine.to(tensor_to_send.device)
+        dests = [d.to(tensor_to_send.device) for d in dests]
+    dist.all_gather(dests, mine, group=cp_group)
+    dests = [int(d.item()) for d in dests]
+    senders = [r for r in range(world) if dests[r] == me and r != me]
+    bufs = [torch.empty_like(tensor_to_send) for _ in senders]
+    sends = [] if dests[me] == me else [(tensor_to_send.contiguous(), members[dests[me]])]
+    for w in exchange(sends, [(b, members[r]) for b, r in zip(bufs, senders)], cp_group):
+        w.wait()
+    total = torch.zeros_like(tensor_to_send)
+    parts = dict(zip(senders, bufs))
+    if dests[me] == me:
+        parts[me] = tensor_to_send
+    for r in sorted(parts):
+        total += parts[r]
+    return total

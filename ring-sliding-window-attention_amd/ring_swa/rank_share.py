@@ -94,24 +94,26 @@ class RankShareFunc(torch.autograd.Function):
     ``[2, batch, seq, kv_heads, dim]`` chunk of rank ``rank - i``."""
 
     @staticmethod
-    def forward(ctx, q, k, v, window_size, cp_size, rank, softmax_scale, ring_dtypes, *prev_kv):
+    def forward(ctx, q, k, v, window_size, cp_size, rank, softmax_scale, ring_dtypes, one_pass,
+                *prev_kv):
         b, s, hq, d = q.shape
         if softmax_scale is None:
             softmax_scale = d ** (-0.5)
         plan = plan_nonvarlen(s, window_size, cp_size, rank)
         for (i, _, _, _, _) in plan:
             assert i == 0 or i <= len(prev_kv), f"step {i} needs the chunk of rank {rank - i}"
-        out, lse = _forward_blocks(q, k, v, prev_kv, plan, softmax_scale, None, ring_dtypes)
+        out, lse = _forward_blocks(q, k, v, prev_kv, plan, softmax_scale, None, ring_dtypes,
+                                   one_pass)
         ctx.save_for_backward(q, k, v, out, lse, *prev_kv)
-        ctx.plan, ctx.scale, ctx.ring_dtypes = plan, softmax_scale, ring_dtypes
+        ctx.plan, ctx.scale, ctx.ring_dtypes, ctx.one_pass = plan, softmax_scale, ring_dtypes, one_pass
         return out
 
     @staticmethod
     def backward(ctx, do):
         q, k, v, out, lse, *prev_kv = ctx.saved_tensors
         grads = _backward_blocks(q, k, v, prev_kv, out, lse, do, ctx.plan, ctx.scale, None,
-                                 ctx.ring_dtypes)
-        return (grads[0], grads[1], grads[2], None, None, None, None, None, *grads[3:])
+                                 ctx.ring_dtypes, ctx.one_pass)
+        return (grads[0], grads[1], grads[2], None, None, None, None, None, None, *grads[3:])
 
 
 _CU_CACHE = {}
@@ -233,10 +235,10 @@ def _one_pass(q, k, v, prev_kv, plan, local_cu):
     return w, kk, vv, tail
 
 
-def _forward_blocks(q, k, v, prev_kv, plan, scale, local_cu, ring_dtypes):
+def _forward_blocks(q, k, v, prev_kv, plan, scale, local_cu, ring_dtypes, one_pass=True):
     """Run the planned blocks and merge them.  Dense 4-d tensors (batch 1 when packed)."""
     assert plan and plan[0][0] == 0, "the diagonal block comes first: it covers every row"
-    one = None if ring_dtypes else _one_pass(q, k, v, prev_kv, plan, local_cu)
+    one = _one_pass(q, k, v, prev_kv, plan, local_cu) if one_pass and not ring_dtypes else None
     if one is not None:
         # One band over [tail of the previous chunk | own chunk]: row i sees the w + 1 keys that
         # end at its own position, wherever the chunk boundary falls -- the sum the two blocks
@@ -267,12 +269,13 @@ def _forward_blocks(q, k, v, prev_kv, plan, scale, local_cu, ring_dtypes):
     return out, lse
 
 
-def _backward_blocks(q, k, v, prev_kv, out, lse, do, plan, scale, local_cu, ring_dtypes=False):
+def _backward_blocks(q, k, v, prev_kv, out, lse, do, plan, scale, local_cu, ring_dtypes=False,
+                     one_pass=True):
     if do.stride(-1) != 1:
         do = do.contiguous()
     assert plan and plan[0][0] == 0
     if len(plan) == 2:
-        one = None if ring_dtypes else _one_pass(q, k, v, prev_kv, plan, local_cu)
+        one = _one_pass(q, k, v, prev_kv, plan, local_cu) if one_pass and not ring_dtypes else None
         if one is not None:
             return _backward_one_pass(q, k, v, prev_kv, out, lse, do, one, scale)
         return _backward_two_blocks(q, k, v, prev_kv, out, lse, do, plan, scale, local_cu)
@@ -400,15 +403,19 @@ def ring_rank_share_attn(
     softmax_scale: Optional[float] = None,
     *,
     ring_dtypes: bool = False,
+    one_pass: bool = True,
 ) -> torch.Tensor:
     """Attention output of rank ``cp_local_rank`` for its chunk ``q, k, v``
     (``[batch, seq, heads, dim]``), given ``prev_kv[i - 1] = stack([k, v])`` of rank
     ``cp_local_rank - i``.  Differentiable w.r.t. ``q, k, v`` and every ``prev_kv``
     entry (the gradient a real ring would send back).  ``ring_dtypes=True`` keeps the
-    running output in fp32 and the running LSE in fp64 as upstream does."""
+    running output in fp32 and the running LSE in fp64 as upstream does.  ``one_pass=False``
+    keeps upstream's block structure -- own-chunk block, previous-chunk block, LSE merge
+    (``ring_swa/sliding_window/nonvarlen.py:95-154``) -- where the default computes the two as
+    one band over both key ranges (window shorter than a chunk)."""
     assert q.shape[1] == k.shape[1] == v.shape[1], "Sequence length must be the same"
     return RankShareFunc.apply(q, k, v, int(window_size), int(cp_size), int(cp_local_rank),
-                               softmax_scale, bool(ring_dtypes), *prev_kv)
+                               softmax_scale, bool(ring_dtypes), bool(one_pass), *prev_kv)
 
 
 def ring_rank_share_attn_varlen(

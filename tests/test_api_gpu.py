@@ -46,6 +46,22 @@ def test_sliding_window_dense():
     _compare(_gpu_fwd_bwd(lambda q, k, v: ring_swa.ring_sliding_window_attn(q, k, v, 100), q, k, v, do), ref)
 
 
+def test_cpu_plumbing_shape_in_16_bits():
+    """The shape of the CPU-runnable configuration -- batch 1, seq 1024, 4 q = 4 kv heads,
+    head_dim 64, window 256, seed 0, scale 1/8, dO ~ N(0,1): the workload the CPU baseline of
+    the benchmark times in fp32 -- through the HIP kernels in bf16 and fp16, against the fp32
+    oracle on the same (rounded) inputs."""
+    import ring_swa
+
+    torch.manual_seed(0)
+    q32, k32, v32, do32 = (torch.randn(1, 1024, 4, 64) for _ in range(4))
+    for dtype in (torch.bfloat16, torch.float16):
+        q, k, v, do = (t.to(dtype) for t in (q32, k32, v32, do32))
+        ref = O.attention_fwd_bwd(lambda q, k, v: O.sliding_window_attn(q, k, v, 256, 1 / 8), q, k, v, do)
+        fn = lambda q, k, v: ring_swa.ring_sliding_window_attn(q, k, v, 256, softmax_scale=1 / 8)  # noqa: E731
+        _compare(_gpu_fwd_bwd(fn, q, k, v, do), ref)
+
+
 def test_sliding_window_varlen_positional_like_upstream_callers():
     import ring_swa
 

@@ -80,15 +80,21 @@ def test_config2_swa_batch2_seq8192_mha_window1000():
     assert torch.equal(q2.grad, qg.grad) and torch.equal(k2.grad, kg.grad) and torch.equal(v2.grad, vg.grad)
 
 
-def test_config3_rank_share_chunk8192_gqa_window4096():
+@pytest.mark.parametrize("route", ["one_pass", "two_blocks", "ring_dtypes"])
+def test_config3_rank_share_chunk8192_gqa_window4096(route):
+    """The three routes of the rank step: one band over [previous chunk's tail | own chunk]
+    (default); own-chunk block + previous-chunk corner block merged in 16 bits (upstream's block
+    structure, ring_swa/sliding_window/nonvarlen.py:95-154); the same two blocks through the
+    accumulating block operators with fp32 output / fp64 LSE (what the ring over a cp_group runs)."""
     import ring_swa
 
+    kw = {"one_pass": {}, "two_blocks": {"one_pass": False}, "ring_dtypes": {"ring_dtypes": True}}[route]
     s, hq, hk, w, cp, rank = 8192, 32, 8, 4096, 8, 1
     q, do = _randn((1, s, hq, D), 0), _randn((1, s, hq, D), 1)
     k, v = _randn((1, s, hk, D), 2), _randn((1, s, hk, D), 3)
     prev = _randn((2, 1, s, hk, D), 4)
     qg, kg, vg, pg = (t.clone().requires_grad_() for t in (q, k, v, prev))
-    out = ring_swa.ring_rank_share_attn(qg, kg, vg, [pg], w, cp, rank)
+    out = ring_swa.ring_rank_share_attn(qg, kg, vg, [pg], w, cp, rank, **kw)
     out.backward(do)
     # the same rows in the global picture: keys = previous chunk then own chunk,
     # queries aligned bottom-right, one causal band of width w

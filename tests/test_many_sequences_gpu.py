@@ -48,9 +48,10 @@ def test_pack_of_many_short_sequences(n_seq, lo, hi, window, sink, d):
         assert relnorm(x, r) <= GRAD_TOL, name
 
 
-def test_pack_of_4096_sequences_runs_at_the_speed_of_its_size():
-    """65 536 tokens as 4096 sequences of 16: about the work of 512 tiles.  A search that
-    walked the sequence list in every block took milliseconds here; bounded generously."""
+def test_pack_of_4096_sequences_equals_its_dense_view():
+    """65 536 tokens as 4096 sequences of 16 (every block has to find its sequence among 4096)
+    against the same problem as a dense [4096, 16] batch: the same bits.  (The time of this
+    pack is a key of the benchmark, not an assertion here.)"""
     from ring_swa.ops import attn_bwd, attn_fwd
 
     n, L, hq, hk, d = 4096, 16, 8, 2, 128
@@ -64,17 +65,8 @@ def test_pack_of_4096_sequences_runs_at_the_speed_of_its_size():
         attn_bwd(q, k, v, out, lse, do, dq, dk, dv, None, (8, 0), True, cu_dev, cu_dev)
         return out
 
-    run()
+    out = run()
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(5):
-        out = run()
-    e1.record()
-    torch.cuda.synchronize()
-    ms = e0.elapsed_time(e1) / 5
-    print(f"4096 x 16 tokens fwd+bwd: {ms:.3f} ms")
-    assert ms < 3.0, ms
     # dense view of the same problem: [4096, 16] batches
     ref, _ = attn_fwd(q.view(n, L, hq, d), k.view(n, L, hk, d), v.view(n, L, hk, d), None, (8, 0),
                       True)

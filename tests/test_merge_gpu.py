@@ -48,6 +48,29 @@ def test_merge_matches_oracle(kind, shape):
     assert torch.equal(don.cpu(), on) and torch.equal(dln.cpu(), ln)
 
 
+def test_merge_at_the_shape_of_the_reference_self_test():
+    """ring_swa/ops/merge.py:211-255: batch 8, seq 8192, 16 heads, head_dim 128, running output
+    fp32 / LSE fp64, new partial bf16 / fp32, all N(0,1); the reference asks atol = rtol = 1e-2
+    on the output and 1e-5 on the LSE.  1 048 576 rows: every block and lane pattern of the
+    kernel at full occupancy, which the small cases do not reach.  (The oracle's formula runs
+    on the device here: fp64 on 67 million elements.)"""
+    from ring_swa.ops import merge_attn_out
+
+    b, s, h, d = 8, 8192, 16, 128
+    g = torch.Generator(device="cuda").manual_seed(0)
+    o = torch.randn(b, s, h, d, generator=g, device="cuda")
+    l = torch.randn(b, h, s, generator=g, device="cuda", dtype=torch.float64)
+    on = torch.randn(b, s, h, d, generator=g, device="cuda").bfloat16()
+    ln = torch.randn(b, h, s, generator=g, device="cuda")
+    ref_o, ref_l = O.merge(o.double(), l, on.double(), ln.double())
+    snap_on, snap_ln = on.clone(), ln.clone()
+    merge_attn_out(o, l, on, ln)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(o.double(), ref_o, atol=2e-6, rtol=2e-6)  # (asked: 1e-2)
+    torch.testing.assert_close(l, ref_l, atol=1e-5, rtol=1e-5)
+    assert torch.equal(on, snap_on) and torch.equal(ln, snap_ln)
+
+
 def test_merge_identity_and_empty_rows():
     from ring_swa.ops import merge_attn_out
 

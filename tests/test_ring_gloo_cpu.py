@@ -62,6 +62,39 @@ def oracle_kernels(dtype=torch.float64):
                            merge=merge)
 
 
+def _check_collective_helpers(rank, world, group):
+    """The three helpers of upstream's streaming-LLM ring (``ops/comm.py:43-149``), by their
+    defining sums: broadcast copies the source's tensor, reduce leaves the sum of all on the
+    destination, the exchange returns the sum of what the ranks that chose this rank sent."""
+    from ring_swa.ops import (broadcast_tensor_to_group, exchange_and_sum_tensors,
+                              reduce_sum_tesnsor_to_rank)
+
+    base = torch.arange(6, dtype=torch.float64).reshape(2, 3)
+    t = base * (rank + 1)
+    broadcast_tensor_to_group(t, world - 1, group).wait()
+    assert torch.equal(t, base * world)
+    t = base + rank
+    out = reduce_sum_tesnsor_to_rank(t, 0, group)
+    if rank == 0:
+        assert out is t and torch.equal(t, base * world + sum(range(world)))
+    # everybody sends to rank 0 except rank 0, which sends to the last rank
+    dest = world - 1 if rank == 0 else 0
+    got = exchange_and_sum_tensors(base * 10 ** rank, dest, group)
+    if rank == 0:
+        want = base * sum(10 ** r for r in range(1, world))
+    elif rank == world - 1:
+        want = base * 1
+    else:
+        want = torch.zeros_like(base)
+    assert torch.equal(got, want), (rank, got, want)
+    # a rank may send to itself; ranks nobody sends to get zeros
+    got = exchange_and_sum_tensors(base + rank, rank if rank % 2 == 0 else rank - 1, group)
+    want = torch.zeros_like(base)
+    if rank % 2 == 0:
+        want = (base + rank) + ((base + rank + 1) if rank + 1 < world else 0)
+    assert torch.equal(got, want), (rank, got, want)
+
+
 def _worker(rank, world, port, cases, results):
     sys.path.insert(0, ROOT)
     sys.path.insert(0, os.path.join(ROOT, "ring-sliding-window-attention_amd"))
@@ -82,6 +115,7 @@ def _worker(rank, world, port, cases, results):
             got = get_group_local_to_global_rank_map(sub)
             assert got == dict(enumerate(sorted(members))) or got == dict(enumerate(members)), got
             assert got[dist.get_rank(sub)] == rank
+    _check_collective_helpers(rank, world, group)
     from ring_swa.ring_slm import ring_slm_attn
 
     K = oracle_kernels()

@@ -20,20 +20,26 @@ def _case(seed, b, s, hq, hk, d, window, packed_cu=None):
     return q, k, v, do
 
 
-def _both(q, k, v, do, window, cu=None):
+def _both(q, k, v, do, window, cu=None, ns=0):
     from ring_swa.ops import attn_bwd, attn_fwd
+    from ring_swa.ops.band_attn import bwd_static_init
 
-    out, lse = attn_fwd(q, k, v, None, window, True, cu, cu)
+    out, lse = attn_fwd(q, k, v, None, window, True, cu, cu, num_sink=ns)
+    bwd_static_init()  # (the one-time address look-up may load the device image: not counted)
     grads = []
     for static in (False, True):
         dq, dk, dv = (torch.full_like(t, float("nan")) for t in (q, k, v))
+        torch.cuda.synchronize()
         before = torch.cuda.memory_allocated()
-        attn_bwd(q, k, v, out, lse, do, dq, dk, dv, None, window, True, cu, cu,
+        free_before = torch.cuda.mem_get_info()[0]  # the device's own count: sees any hipMalloc
+        attn_bwd(q, k, v, out, lse, do, dq, dk, dv, None, window, True, cu, cu, num_sink=ns,
                  static_workspace=static)
+        torch.cuda.synchronize()
         if static:
             assert torch.cuda.memory_allocated() == before, "the static entry point allocated"
+            assert torch.cuda.mem_get_info()[0] == free_before, (
+                "device memory was allocated under the static entry point")
         grads.append((dq, dk, dv))
-    torch.cuda.synchronize()
     return grads
 
 
@@ -63,6 +69,53 @@ def test_static_backward_equals_workspace_backward_twice_in_a_row():
     q, k, v, do = _case(1, 1, 700, 4, 4, 64, (64, 0), packed_cu=cu)
     (a, b) = _both(q, k, v, do, (64, 0), cu)
     _same(a, b)
+
+
+def test_static_backward_with_sink_keys_under_a_bounded_window():
+    """Then the sink kernel's arrival counters and fp32 sums live in the built-in buffer too
+    (dense, then packed and smaller): the counters must come back to zero between the calls."""
+    q, k, v, do = _case(2, 2, 1100, 8, 2, 128, (100, 0))
+    k[:, :3] *= 4
+    _same(*_both(q, k, v, do, (100, 0), ns=3))
+    cu = torch.tensor([0, 300, 301, 900], dtype=torch.int32, device="cuda")
+    q, k, v, do = _case(3, 1, 900, 4, 2, 64, (40, 0), packed_cu=cu)
+    _same(*_both(q, k, v, do, (40, 0), cu, ns=5))
+    _same(*_both(q, k, v, do, (40, 0), cu, ns=5))
+
+
+def test_static_backward_replays_from_a_graph():
+    """For callers under HIP graph capture: warm up (address look-up) outside the capture, capture
+    one static backward, replay it with eager work in between, same bits as the eager call."""
+    from ring_swa.ops import attn_bwd, attn_fwd
+    from ring_swa.ops.band_attn import bwd_static_init
+
+    q, k, v, do = _case(4, 1, 768, 8, 2, 128, (200, 0))
+    out, lse = attn_fwd(q, k, v, None, (200, 0), True)
+    dq, dk, dv = (torch.empty_like(t) for t in (q, k, v))
+    run = lambda: attn_bwd(q, k, v, out, lse, do, dq, dk, dv, None, (200, 0), True,  # noqa: E731
+                           static_workspace=True)
+    bwd_static_init()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        run()
+    for trial in range(3):
+        g = torch.Generator().manual_seed(20 + trial)
+        do.copy_(torch.randn(do.shape, generator=g).bfloat16())
+        for t in (dq, dk, dv):
+            t.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in (dq, dk, dv)]
+        run()  # eager work between the replays
+        torch.cuda.synchronize()
+        for a, b in zip(got, (dq, dk, dv)):
+            assert torch.equal(a, b), f"replay {trial} differs from the eager call"
 
 
 def test_static_backward_refuses_sizes_beyond_its_buffer():
