@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define RSWA_VERSION 2
+#define RSWA_VERSION 3
 
 typedef enum rswa_status {
   RSWA_OK = 0,
@@ -212,7 +212,29 @@ typedef struct rswa_attn_params {
    * have run before it.  rswa_attn_bwd_static never uses it.  Same interface replaced:
    * ring_swa/ops/wrap_flash.py:276-429. */
   int32_t ds_handoff;
+  /* Accumulators of the ring loops (ring_swa/sliding_window/nonvarlen.py:53-59, 203-206: fp32
+   * running output, fp64 running LSE, fp32 dq and dkv that every block is added to) taken as
+   * they are, so that a block needs no temporary, no merge launch and no elementwise passes
+   * (ring_swa/ops/attn.py:23-37, ring_swa/sliding_window/nonvarlen.py:318-321).  Bit mask:
+   *   RSWA_WIDE_OUT  forward: out is fp32 and lse is fp64 (strides in their own elements).  The
+   *                  block's output is rounded to the 16-bit type of q first, as the reference's
+   *                  block kernel returns it, then written as fp32 -- or, with out_accumulate,
+   *                  merged into what out / lse hold: the bits of rswa_attn_fwd into 16-bit
+   *                  temporaries followed by rswa_merge_attn_out on these accumulators.
+   *   RSWA_WIDE_DQ   backward: dq is fp32: the block's dq, rounded to 16 bits, is written as
+   *                  fp32 or, with dq_accumulate, added to what dq holds.
+   *   RSWA_WIDE_DKV  backward: dk and dv (dk2 / dv2 too) are fp32, written likewise; with
+   *                  dkv_accumulate != 0 the block's values are added to what they hold.  Not
+   *                  with sink keys under a bounded window (RSWA_ERR_UNSUPPORTED).
+   * The backward still reads out in the 16-bit type and lse as fp32 (the reference casts its
+   * accumulators before the backward, ring_swa/sliding_window/nonvarlen.py:156-157). */
+  int32_t wide;
+  int32_t dkv_accumulate; /* only with RSWA_WIDE_DKV */
 } rswa_attn_params;
+
+#define RSWA_WIDE_OUT 1
+#define RSWA_WIDE_DQ 2
+#define RSWA_WIDE_DKV 4
 
 #define RSWA_ADDR_AUTO 0
 #define RSWA_ADDR_FAR 1

@@ -98,10 +98,10 @@ BwdLayout bwd_layout(const rswa_attn_params* p, bool allow_split, bool allow_han
 
 uint64_t bwd_workspace_bytes(const rswa_attn_params* p) { return bwd_layout(p, true, true).total_bytes; }
 
-static bool rows_aligned(const void* ptr, const int64_t* st) {
+static bool rows_aligned(const void* ptr, const int64_t* st, int elem_bytes = 2) {
   if (((uintptr_t)ptr) % 16) return false;
   for (int i = 0; i < 3; i++)
-    if (st[i] % 8) return false;
+    if (st[i] % (16 / elem_bytes)) return false;
   return true;
 }
 
@@ -129,10 +129,15 @@ int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a, bool allow_
                  "attn: totals out of range");
   }
   RSWA_REQUIRE(p->q && p->k && p->v && p->out && p->lse, RSWA_ERR_INVALID, "attn: null tensor");
+  RSWA_REQUIRE((p->wide & ~(RSWA_WIDE_OUT | RSWA_WIDE_DQ | RSWA_WIDE_DKV)) == 0, RSWA_ERR_INVALID,
+               "attn: unknown bits in wide (%d)", p->wide);
+  const bool wide_out = !backward && (p->wide & RSWA_WIDE_OUT);
   RSWA_REQUIRE(rows_aligned(p->q, p->q_stride) && rows_aligned(p->k, p->k_stride) &&
-                   rows_aligned(p->v, p->v_stride) && rows_aligned(p->out, p->out_stride),
+                   rows_aligned(p->v, p->v_stride) &&
+                   rows_aligned(p->out, p->out_stride, wide_out ? 4 : 2),
                RSWA_ERR_UNSUPPORTED, "attn: q/k/v/out rows must start 16-byte aligned");
-  RSWA_REQUIRE(((uintptr_t)p->lse) % 4 == 0, RSWA_ERR_UNSUPPORTED, "attn: lse misaligned");
+  RSWA_REQUIRE(((uintptr_t)p->lse) % (wide_out ? 8 : 4) == 0, RSWA_ERR_UNSUPPORTED,
+               "attn: lse misaligned");
   {
     // Tiles are fetched through 32-bit byte offsets.  The rows of one tile (at most
     // kMaxTileRows) must span less than 2 GiB; when a whole sequence does too, offsets count
@@ -236,6 +241,14 @@ int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a, bool allow_
   a.shift_val = p->shift;
   a.dq_accumulate = backward && p->dq_accumulate != 0;
   a.out_accumulate = !backward && p->out_accumulate != 0;
+  a.wide_out = wide_out;
+  a.wide_dq = backward && (p->wide & RSWA_WIDE_DQ);
+  a.wide_dkv = backward && (p->wide & RSWA_WIDE_DKV);
+  a.dkv_accumulate = a.wide_dkv && p->dkv_accumulate != 0;
+  RSWA_REQUIRE(!(backward && p->dkv_accumulate && !a.wide_dkv), RSWA_ERR_INVALID,
+               "attn_bwd: dkv_accumulate needs fp32 dk / dv (RSWA_WIDE_DKV)");
+  RSWA_REQUIRE(!(a.wide_dkv && p->num_sink > 0 && a.wl >= 0), RSWA_ERR_UNSUPPORTED,
+               "attn_bwd: fp32 dk / dv (RSWA_WIDE_DKV) with sink keys under a bounded window");
   a.n_tile = 0;
   a.n_work = 0;
   {
@@ -268,8 +281,10 @@ int fill_args(const rswa_attn_params* p, bool backward, AttnArgs& a, bool allow_
 
   if (backward) {
     RSWA_REQUIRE(p->dout && p->dq && p->dk && p->dv, RSWA_ERR_INVALID, "attn_bwd: null tensor");
-    RSWA_REQUIRE(rows_aligned(p->dout, p->dout_stride) && rows_aligned(p->dq, p->dq_stride) &&
-                     rows_aligned(p->dk, p->dk_stride) && rows_aligned(p->dv, p->dv_stride),
+    RSWA_REQUIRE(rows_aligned(p->dout, p->dout_stride) &&
+                     rows_aligned(p->dq, p->dq_stride, a.wide_dq ? 4 : 2) &&
+                     rows_aligned(p->dk, p->dk_stride, a.wide_dkv ? 4 : 2) &&
+                     rows_aligned(p->dv, p->dv_stride, a.wide_dkv ? 4 : 2),
                  RSWA_ERR_UNSUPPORTED, "attn_bwd: dout/dq/dk/dv rows must start 16-byte aligned");
     RSWA_REQUIRE(p->dout_stride[1] >= 0 && p->dout_stride[1] * 2 < ((1ll << 31) - 65536) / kMaxTileRows,
                  RSWA_ERR_UNSUPPORTED, "attn_bwd: row stride of dout is negative or too large");

@@ -52,6 +52,38 @@
 namespace rswa {
 namespace {
 
+// One lane's 8 consecutive values of a gradient row, already rounded to the 16-bit type, into
+// the caller's buffer at element offset `at`: as they are, as fp32 (a ring accumulator), and in
+// either case added to what the buffer holds (fp32 sum, one rounding for a 16-bit buffer).
+template <typename T>
+__device__ __forceinline__ void put_grad8(void* buf, int64_t at, typename Mma<T>::V8 val, bool wide,
+                                          bool accumulate) {
+  using V8 = typename Mma<T>::V8;
+  if (wide) {
+    float* dst = (float*)buf + at;
+    f32x4 y[2];
+#pragma unroll
+    for (int hh = 0; hh < 2; hh++) {
+      f32x4 old = {0.f, 0.f, 0.f, 0.f};
+      if (accumulate) old = *(const f32x4*)(dst + 4 * hh);
+#pragma unroll
+      for (int j = 0; j < 4; j++) y[hh][j] = old[j] + (float)val[4 * hh + j];
+    }
+    *(f32x4*)dst = y[0];
+    *(f32x4*)(dst + 4) = y[1];
+  } else {
+    T* dst = (T*)buf + at;
+    if (accumulate) {
+      const V8 old = *(const V8*)dst;
+      float sum[8];
+#pragma unroll
+      for (int j = 0; j < 8; j++) sum[j] = (float)old[j] + (float)val[j];
+      val = Mma<T>::pack(sum);
+    }
+    *(V8*)dst = val;
+  }
+}
+
 // ============================================================================
 // dK / dV
 // ============================================================================
@@ -128,8 +160,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
   const int64_t seg_row0 = seg2 ? -(int64_t)a.seg : s.k_row0;
   const T* k_ptr = (const T*)(seg2 ? a.k2 : a.k) + b * a.k_st[0] + seg_row0 * a.k_st[1] + hk * a.k_st[2];
   const T* v_ptr = (const T*)(seg2 ? a.v2 : a.v) + b * a.v_st[0] + seg_row0 * a.v_st[1] + hk * a.v_st[2];
-  T* dk_ptr = (T*)(seg2 ? a.dk2 : a.dk) + b * a.dk_st[0] + seg_row0 * a.dk_st[1] + hk * a.dk_st[2];
-  T* dv_ptr = (T*)(seg2 ? a.dv2 : a.dv) + b * a.dv_st[0] + seg_row0 * a.dv_st[1] + hk * a.dv_st[2];
+  // (gradient buffers: T or, as ring accumulators, fp32 -- element offsets)
+  void* const dk_buf = seg2 ? a.dk2 : a.dk;
+  void* const dv_buf = seg2 ? a.dv2 : a.dv;
+  const int64_t dk_off = b * a.dk_st[0] + seg_row0 * a.dk_st[1] + hk * a.dk_st[2];
+  const int64_t dv_off = b * a.dv_st[0] + seg_row0 * a.dv_st[1] + hk * a.dv_st[2];
   const int64_t ws_row0 = a.cu_q ? s.q_row0 : (int64_t)b * a.seqlen_q;
 
   // ---- query tiles that can see this key tile -------------------------------
@@ -542,9 +577,17 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
     const int jc = jw0 + kb * 32 + l32_e;
     if (jc < len_k) {
       const float sc = mtx == 0 ? a.scale : 1.f;
-      T* dst = mtx == 0 ? dk_ptr + (int64_t)jc * a.dk_st[1] : dv_ptr + (int64_t)jc * a.dv_st[1];
-      *(typename M::V4*)(dst + d * 32 + 8 * i4 + 4 * g_e) =
-          M::pack4(val[0] * sc, val[1] * sc, val[2] * sc, val[3] * sc);
+      const int64_t at = (mtx == 0 ? dk_off + (int64_t)jc * a.dk_st[1] : dv_off + (int64_t)jc * a.dv_st[1]) +
+                         d * 32 + 8 * i4 + 4 * g_e;
+      const typename M::V4 h4 = M::pack4(val[0] * sc, val[1] * sc, val[2] * sc, val[3] * sc);
+      if (a.wide_dkv) {
+        float* dst = (float*)(mtx == 0 ? dk_buf : dv_buf) + at;
+        f32x4 y = {(float)h4[0], (float)h4[1], (float)h4[2], (float)h4[3]};
+        if (a.dkv_accumulate) y += *(const f32x4*)dst;
+        *(f32x4*)dst = y;
+      } else {
+        *(typename M::V4*)((T*)(mtx == 0 ? dk_buf : dv_buf) + at) = h4;
+      }
     }
   };
   // Without a split (SPLIT = false, nsplit = 1) the lane's sums go straight out.  Otherwise the
@@ -580,7 +623,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
                          acc[4 * i4 + 3] * sc);
           }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wave's own writes have landed
-        T* dst = mtx == 0 ? dk_ptr : dv_ptr;
+        void* const dst = mtx == 0 ? dk_buf : dv_buf;
+        const int64_t dst_off = mtx == 0 ? dk_off : dv_off;
         const int64_t dst_st = mtx == 0 ? a.dk_st[1] : a.dv_st[1];
 #pragma unroll
         for (int n = 0; n < 32 * C::CPR / 64; n++) {
@@ -588,7 +632,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnArgs a) {
           const int row = idx / C::CPR, c = idx % C::CPR;
           const V8 val = *(const V8*)(stage + row * C::ROWB + ((c ^ (row & (C::CPR - 1))) << 4));
           const int jc = jw0 + kb * 32 + row;
-          if (jc < len_k) *(V8*)(dst + (int64_t)jc * dst_st + c * 8) = val;
+          if (jc < len_k)
+            put_grad8<T>(dst, dst_off + (int64_t)jc * dst_st + c * 8, val, a.wide_dkv, a.dkv_accumulate);
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // read before the next block overwrites
       }
@@ -933,7 +978,7 @@ void attn_bwd_dq_kernel(const AttnArgs a) {
   const T* do_ptr = (const T*)a.dout + b * a.do_st[0] + s.q_row0 * a.do_st[1] + hq * a.do_st[2];
   const T* k_ptr = (const T*)a.k + b * a.k_st[0] + s.k_row0 * a.k_st[1] + hk * a.k_st[2];
   const T* v_ptr = (const T*)a.v + b * a.v_st[0] + s.k_row0 * a.v_st[1] + hk * a.v_st[2];
-  T* dq_ptr = (T*)a.dq + b * a.dq_st[0] + s.q_row0 * a.dq_st[1] + hq * a.dq_st[2];
+  const int64_t dq_off = b * a.dq_st[0] + s.q_row0 * a.dq_st[1] + hq * a.dq_st[2];  // (T or fp32)
   const int64_t ws_row0 = a.cu_q ? s.q_row0 : (int64_t)b * a.seqlen_q;
 
   // ---- key tiles this block visits (same rule as the forward kernel) -----------
@@ -1159,16 +1204,9 @@ void attn_bwd_dq_kernel(const AttnArgs a) {
         const int c = lane + n * 64;
         const int row = c / C::CPR, col = (c % C::CPR) * 8;
         if (r0 + row < len_q) {
-          V8 val = *(const V8*)(stage + row * C::O_STRIDE + col * 2);
-          T* dst = dq_ptr + (int64_t)(r0 + row) * a.dq_st[1] + col;
-          if (a.dq_accumulate) {
-            const V8 old = *(const V8*)dst;
-            float sum[8];
-#pragma unroll
-            for (int j = 0; j < 8; j++) sum[j] = (float)old[j] + (float)val[j];
-            val = M::pack(sum);
-          }
-          *(V8*)dst = val;
+          const V8 val = *(const V8*)(stage + row * C::O_STRIDE + col * 2);
+          put_grad8<T>(a.dq, dq_off + (int64_t)(r0 + row) * a.dq_st[1] + col, val, a.wide_dq,
+                       a.dq_accumulate);
         }
       }
     }
@@ -1263,7 +1301,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_ds_kernel(const AttnArgs a) {
 
   const T* k_ptr = (const T*)a.k + b * a.k_st[0] + s.k_row0 * a.k_st[1] + hk * a.k_st[2];
   const T* k2_ptr = a.k2 ? (const T*)a.k2 + b * a.k_st[0] + hk * a.k_st[2] : k_ptr;
-  T* dq_ptr = (T*)a.dq + b * a.dq_st[0] + s.q_row0 * a.dq_st[1] + hq * a.dq_st[2];
+  const int64_t dq_off = b * a.dq_st[0] + s.q_row0 * a.dq_st[1] + hq * a.dq_st[2];  // (T or fp32)
 
   // ---- key stages of the block (64 keys each): those any of its rows can see -------------
   const int i_last = min(i0 + bm, len_q) - 1;
@@ -1414,18 +1452,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_ds_kernel(const AttnArgs a) {
     for (int n = 0; n < 32 * C::CPR / 64; n++) {
       const int cc = lane + n * 64;
       const int row = cc / C::CPR, col = (cc % C::CPR) * 8;
-      V8 val = *(const V8*)(stg + row * C::O_STRIDE + col * 2);
-      if (r0 + 32 * t + row < len_q) {
-        T* dst = dq_ptr + (int64_t)(r0 + 32 * t + row) * a.dq_st[1] + col;
-        if (a.dq_accumulate) {
-          const V8 old = *(const V8*)dst;
-          float sum[8];
-#pragma unroll
-          for (int j = 0; j < 8; j++) sum[j] = (float)old[j] + (float)val[j];
-          val = M::pack(sum);
-        }
-        *(V8*)dst = val;
-      }
+      const V8 val = *(const V8*)(stg + row * C::O_STRIDE + col * 2);
+      if (r0 + 32 * t + row < len_q)
+        put_grad8<T>(a.dq, dq_off + (int64_t)(r0 + 32 * t + row) * a.dq_st[1] + col, val, a.wide_dq,
+                     a.dq_accumulate);
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   }
@@ -1436,9 +1466,23 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_ds_kernel(const AttnArgs a) {
 // rows: -inf, so that P = exp2(S*c - lse2) is zero).  One 16-lane (D=128) or 8-lane (D=64) group per
 // (row, head).
 // ============================================================================
+// A block owns PrepCfg::ROWS consecutive rows of one q head -- the statistics, [head][row], are then
+// written as whole cache lines -- and neighbouring blocks take neighbouring heads, so that the
+// blocks in flight sweep out / dout as one dense front; all eight loads of a thread's four rows
+// are issued before the first use (one row per thread and the heads innermost: 39 -> 27 us on
+// 8192 rows x 32 heads, head_dim 128).
+template <int D>
+struct PrepCfg {
+  static constexpr int LPR = D / 8;         // lanes per row
+  static constexpr int RP = 256 / LPR;      // rows per pass
+  static constexpr int NR = 4;              // passes
+  static constexpr int ROWS = RP * NR;      // rows per block
+};
+
 template <typename T, int D>
 __global__ __launch_bounds__(256) void attn_bwd_prep_kernel(const AttnArgs a) {
-  constexpr int LPR = D / 8;
+  using P = PrepCfg<D>;
+  using V8 = typename Mma<T>::V8;
   // arrival counters of the dK/dV kernel's split blocks start from zero
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < a.n_count; i += (int64_t)gridDim.x * 256)
     a.dkv_count[i] = 0;
@@ -1449,44 +1493,49 @@ __global__ __launch_bounds__(256) void attn_bwd_prep_kernel(const AttnArgs a) {
     const int64_t used = a.rows_q * a.heads_q;
     if (used + threadIdx.x < a.delta - a.lse2) a.lse2[used + threadIdx.x] = -__builtin_inff();
   }
-  const int64_t unit = ((int64_t)blockIdx.x * 256 + threadIdx.x) / LPR;  // (row, head)
-  const int c = (threadIdx.x % LPR) * 8;
-  if (unit >= a.rows_q * a.heads_q) return;
-  const int h = (int)(unit % a.heads_q);
-  const int64_t row = unit / a.heads_q;
-  int64_t o_off, do_off, l_off;
-  if (a.cu_q) {
-    o_off = row * a.o_st[1];
-    do_off = row * a.do_st[1];
-    l_off = row * a.lse_st[2];
-  } else {
-    const int64_t bb = row / a.seqlen_q, i = row % a.seqlen_q;
-    o_off = bb * a.o_st[0] + i * a.o_st[1];
-    do_off = bb * a.do_st[0] + i * a.do_st[1];
-    l_off = bb * a.lse_st[0] + i * a.lse_st[2];
-  }
+  const int h = (int)(blockIdx.x % (unsigned)a.heads_q);
+  const int64_t row0 = (int64_t)(blockIdx.x / (unsigned)a.heads_q) * P::ROWS + threadIdx.x / P::LPR;
+  const int c = (threadIdx.x % P::LPR) * 8;
   // Packed rows past the last sequence belong to nobody: their out / dout may hold anything
   // (NaN included), and the tile kernels read the statistics of the rows that follow a
   // sequence's last tile.  They get the neutral pair, which keeps P and dS exactly zero.
-  if (a.cu_q && row >= a.cu_q[a.batch]) {
-    if (c == 0) {
-      a.delta[(int64_t)h * a.rows_q + row] = 0.f;
-      a.lse2[(int64_t)h * a.rows_q + row] = -__builtin_inff();
+  const int64_t rows_real = a.cu_q ? (int64_t)a.cu_q[a.batch] : a.rows_q;
+  V8 o8[P::NR], d8[P::NR];
+  float l[P::NR];
+#pragma unroll
+  for (int i = 0; i < P::NR; i++) {
+    const int64_t row = row0 + i * P::RP;
+    o8[i] = d8[i] = V8{0, 0, 0, 0, 0, 0, 0, 0};
+    l[i] = -__builtin_inff();
+    if (row < rows_real) {
+      int64_t o_off, do_off, l_off;
+      if (a.cu_q) {
+        o_off = row * a.o_st[1];
+        do_off = row * a.do_st[1];
+        l_off = row * a.lse_st[2];
+      } else {
+        const int64_t bb = row / a.seqlen_q, ii = row % a.seqlen_q;
+        o_off = bb * a.o_st[0] + ii * a.o_st[1];
+        do_off = bb * a.do_st[0] + ii * a.do_st[1];
+        l_off = bb * a.lse_st[0] + ii * a.lse_st[2];
+      }
+      o8[i] = *(const V8*)((const T*)a.out + o_off + h * a.o_st[2] + c);
+      d8[i] = *(const V8*)((const T*)a.dout + do_off + h * a.do_st[2] + c);
+      if (c == 0) l[i] = a.lse[l_off + h * a.lse_st[1]];
     }
-    return;
   }
-  using V8 = typename Mma<T>::V8;
-  const V8 o8 = *(const V8*)((const T*)a.out + o_off + h * a.o_st[2] + c);
-  const V8 d8 = *(const V8*)((const T*)a.dout + do_off + h * a.do_st[2] + c);
-  float acc = 0.f;
 #pragma unroll
-  for (int j = 0; j < 8; j++) acc += (float)o8[j] * (float)d8[j];
+  for (int i = 0; i < P::NR; i++) {
+    const int64_t row = row0 + i * P::RP;
+    float acc = 0.f;
 #pragma unroll
-  for (int m = LPR / 2; m >= 1; m >>= 1) acc += __shfl_xor(acc, m, 64);
-  if (c == 0) {
-    a.delta[(int64_t)h * a.rows_q + row] = -acc;
-    const float l = a.lse[l_off + h * a.lse_st[1]];
-    a.lse2[(int64_t)h * a.rows_q + row] = (l == -__builtin_inff()) ? l : -l * kLog2e;
+    for (int j = 0; j < 8; j++) acc += (float)o8[i][j] * (float)d8[i][j];
+#pragma unroll
+    for (int m = P::LPR / 2; m >= 1; m >>= 1) acc += __shfl_xor(acc, m, 64);
+    if (c == 0 && row < a.rows_q) {
+      a.delta[(int64_t)h * a.rows_q + row] = -acc;  // (rows nobody owns: -0)
+      a.lse2[(int64_t)h * a.rows_q + row] = (l[i] == -__builtin_inff()) ? l[i] : -l[i] * kLog2e;
+    }
   }
 }
 
@@ -1515,9 +1564,10 @@ template <typename T, int D>
 int launch_bwd(AttnArgs& a, hipStream_t stream, int phases) {
   const int64_t units = a.rows_q * a.heads_q;
   if (units > 0 && (phases & RSWA_BWD_PREP)) {
-    const unsigned blocks = (unsigned)ceil_div(units * (D / 8), 256);
+    const int64_t blocks = ceil_div(a.rows_q, PrepCfg<D>::ROWS) * a.heads_q;
+    RSWA_REQUIRE(blocks < (1ll << 31), RSWA_ERR_UNSUPPORTED, "attn_bwd: too many (row, head) pairs");
     clear_launch_error();
-    hipLaunchKernelGGL((attn_bwd_prep_kernel<T, D>), dim3(blocks), dim3(256), 0, stream, a);
+    hipLaunchKernelGGL((attn_bwd_prep_kernel<T, D>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
     int rc = check_launch("attn_bwd prep");
     if (rc != RSWA_OK) return rc;
   }

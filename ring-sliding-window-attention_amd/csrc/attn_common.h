@@ -51,6 +51,9 @@ struct AttnArgs {
   int32_t shift_explicit, shift_val;
   int32_t dq_accumulate;  // backward: add to dq instead of overwriting it
   int32_t out_accumulate;  // forward: merge the block into what out / lse hold
+  // fp32 / fp64 accumulators of the ring loops in place of 16-bit / fp32 results (RSWA_WIDE_*):
+  // forward out fp32 + lse fp64; backward dq fp32; backward dk, dv fp32 (+ add to them)
+  int32_t wide_out, wide_dq, wide_dkv, dkv_accumulate;
   int32_t n_tile;          // tiles per sequence (dense) / total tile slots (packed)
   int32_t n_work;          // logical blocks
   // Blocks are dispatched in logical order; these flags reverse the order of the query

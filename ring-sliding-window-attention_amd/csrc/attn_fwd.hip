@@ -94,8 +94,9 @@ void attn_fwd_kernel(const AttnArgs a) {
   const T* q_ptr = (const T*)a.q + b * a.q_st[0] + s.q_row0 * a.q_st[1] + hq * a.q_st[2];
   const T* k_ptr = (const T*)a.k + b * a.k_st[0] + s.k_row0 * a.k_st[1] + hk * a.k_st[2];
   const T* v_ptr = (const T*)a.v + b * a.v_st[0] + s.k_row0 * a.v_st[1] + hk * a.v_st[2];
-  T* o_ptr = (T*)a.out + b * a.o_st[0] + s.q_row0 * a.o_st[1] + hq * a.o_st[2];
-  float* lse_ptr = a.lse + b * a.lse_st[0] + hq * a.lse_st[1] + s.q_row0 * a.lse_st[2];
+  // (element offsets: out is T or, as a ring accumulator, fp32; lse is fp32 or fp64)
+  const int64_t o_off = b * a.o_st[0] + s.q_row0 * a.o_st[1] + hq * a.o_st[2];
+  const int64_t lse_off = b * a.lse_st[0] + hq * a.lse_st[1] + s.q_row0 * a.lse_st[2];
 
   // ---- key tiles this block visits -----------------------------------------
   const int i_last = min(i0 + bm, len_q) - 1;
@@ -350,15 +351,21 @@ void attn_fwd_kernel(const AttnArgs a) {
     const float ninf = -__builtin_inff();
     float lse_new = l_tot > 0.f ? m_run * a.scale + __logf(l_tot) : ninf;
     float w_old = 0.f, w_new = 1.f;
+    const int64_t lse_at = lse_off + (int64_t)iq * a.lse_st[2];
     if (a.out_accumulate && iq < len_q) {
-      const float la = lse_ptr[(int64_t)iq * a.lse_st[2]], lb = lse_new;
+      // (an fp64 running LSE enters the arithmetic as fp32, as in the merge kernel)
+      const float la = a.wide_out ? (float)((const double*)a.lse)[lse_at] : a.lse[lse_at];
+      const float lb = lse_new;
       const bool both_empty = (la == ninf) && (lb == ninf);
       const float diff = both_empty ? 0.f : lb - la;
       w_old = both_empty ? 0.f : 1.f / (1.f + __expf(diff));
       w_new = both_empty ? 0.f : 1.f / (1.f + __expf(-diff));
       lse_new = both_empty ? ninf : fmaxf(la, lb) + log1pf(__expf(-fabsf(diff)));
     }
-    if (g == 0 && iq < len_q) lse_ptr[(int64_t)iq * a.lse_st[2]] = lse_new;
+    if (g == 0 && iq < len_q) {
+      if (a.wide_out) ((double*)a.lse)[lse_at] = (double)lse_new;
+      else a.lse[lse_at] = lse_new;
+    }
     // (the staging buffer is the wave's own: its writes only have to land before its reads)
 #pragma unroll
     for (int d = 0; d < C::DBLK; d++)
@@ -379,21 +386,42 @@ void attn_fwd_kernel(const AttnArgs a) {
       const int row = c / C::CPR, col = (c % C::CPR) * 8;
       if (r0 + row < len_q) {
         V8 val = *(const V8*)(stage + row * C::O_STRIDE + col * 2);
-        T* dst = o_ptr + (int64_t)(r0 + row) * a.o_st[1] + col;
-        if (a.out_accumulate) {
-          const float wo = wgt[2 * row], wn = wgt[2 * row + 1];
-          const V8 old = *(const V8*)dst;
-          float y[8];
+        const int64_t at = o_off + (int64_t)(r0 + row) * a.o_st[1] + col;
+        const float wo = a.out_accumulate ? wgt[2 * row] : 0.f;
+        const float wn = a.out_accumulate ? wgt[2 * row + 1] : 1.f;
+        if (a.wide_out) {
+          // fp32 accumulator: the block's 16-bit values as fp32, or merged into what it holds
+          float* dst = (float*)a.out + at;
+          f32x4 y[2];
 #pragma unroll
-          for (int j = 0; j < 8; j++) {
-            // a zero weight must annihilate whatever the other side holds
-            const float t0 = (wo == 0.f) ? 0.f : (float)old[j] * wo;
-            const float t1 = (wn == 0.f) ? 0.f : (float)val[j] * wn;
-            y[j] = t0 + t1;
+          for (int hh = 0; hh < 2; hh++) {
+            f32x4 old = {0.f, 0.f, 0.f, 0.f};
+            if (a.out_accumulate) old = *(const f32x4*)(dst + 4 * hh);
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+              const float t0 = (wo == 0.f) ? 0.f : old[j] * wo;
+              const float t1 = (wn == 0.f) ? 0.f : (float)val[4 * hh + j] * wn;
+              y[hh][j] = t0 + t1;
+            }
           }
-          val = M::pack(y);
+          *(f32x4*)dst = y[0];
+          *(f32x4*)(dst + 4) = y[1];
+        } else {
+          T* dst = (T*)a.out + at;
+          if (a.out_accumulate) {
+            const V8 old = *(const V8*)dst;
+            float y[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+              // a zero weight must annihilate whatever the other side holds
+              const float t0 = (wo == 0.f) ? 0.f : (float)old[j] * wo;
+              const float t1 = (wn == 0.f) ? 0.f : (float)val[j] * wn;
+              y[j] = t0 + t1;
+            }
+            val = M::pack(y);
+          }
+          *(V8*)dst = val;
         }
-        *(V8*)dst = val;
       }
     }
   }

@@ -27,11 +27,13 @@ struct MergeArgs {
   int32_t lse_f64, lsen_f64;
 };
 
-template <typename T>
-struct Vec8;
+// E = 8 or 4 consecutive elements of a row, to / from fp32 registers, with non-temporal accesses
+// of 16 bytes where the type allows (8 bytes for four 16-bit elements).
+template <typename T, int E>
+struct Vec;
 
 template <>
-struct Vec8<float> {
+struct Vec<float, 8> {
   static __device__ __forceinline__ void load(const float* p, float (&x)[8]) {
     f32x4 a = __builtin_nontemporal_load((const f32x4*)p);
     f32x4 b = __builtin_nontemporal_load((const f32x4*)p + 1);
@@ -50,7 +52,20 @@ struct Vec8<float> {
 };
 
 template <>
-struct Vec8<__bf16> {
+struct Vec<float, 4> {
+  static __device__ __forceinline__ void load(const float* p, float (&x)[4]) {
+    f32x4 a = __builtin_nontemporal_load((const f32x4*)p);
+#pragma unroll
+    for (int i = 0; i < 4; i++) x[i] = a[i];
+  }
+  static __device__ __forceinline__ void store(float* p, const float (&x)[4]) {
+    f32x4 a = {x[0], x[1], x[2], x[3]};
+    __builtin_nontemporal_store(a, (f32x4*)p);
+  }
+};
+
+template <>
+struct Vec<__bf16, 8> {
   static __device__ __forceinline__ void load(const __bf16* p, float (&x)[8]) {
     u32x4 a = __builtin_nontemporal_load((const u32x4*)p);
 #pragma unroll
@@ -67,7 +82,24 @@ struct Vec8<__bf16> {
 };
 
 template <>
-struct Vec8<_Float16> {
+struct Vec<__bf16, 4> {
+  static __device__ __forceinline__ void load(const __bf16* p, float (&x)[4]) {
+    u32x2 a = __builtin_nontemporal_load((const u32x2*)p);
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      x[2 * i] = __uint_as_float(a[i] << 16);
+      x[2 * i + 1] = __uint_as_float(a[i] & 0xffff0000u);
+    }
+  }
+  static __device__ __forceinline__ void store(__bf16* p, const float (&x)[4]) {
+    f32x4 f = {x[0], x[1], x[2], x[3]};
+    bf16x4 h = __builtin_convertvector(f, bf16x4);
+    __builtin_nontemporal_store(h, (bf16x4*)p);
+  }
+};
+
+template <>
+struct Vec<_Float16, 8> {
   static __device__ __forceinline__ void load(const _Float16* p, float (&x)[8]) {
     f16x8 a = __builtin_nontemporal_load((const f16x8*)p);
 #pragma unroll
@@ -80,12 +112,40 @@ struct Vec8<_Float16> {
   }
 };
 
-constexpr int kThreads = 256;
-constexpr int kRowsPerThread = 4;
+template <>
+struct Vec<_Float16, 4> {
+  static __device__ __forceinline__ void load(const _Float16* p, float (&x)[4]) {
+    f16x4 a = __builtin_nontemporal_load((const f16x4*)p);
+#pragma unroll
+    for (int i = 0; i < 4; i++) x[i] = (float)a[i];
+  }
+  static __device__ __forceinline__ void store(_Float16* p, const float (&x)[4]) {
+    f32x4 f = {x[0], x[1], x[2], x[3]};
+    f16x4 h = __builtin_convertvector(f, f16x4);
+    __builtin_nontemporal_store(h, (f16x4*)p);
+  }
+};
 
-// LPR = lanes per row (power of two, LPR * 8 >= head_dim).
+constexpr int kThreads = 256;
+
+// A lane moves E consecutive elements of a row: 8 when the running output is a 16-bit type (16
+// bytes of it a lane), 4 when it is fp32 -- 16 bytes a lane again, so that the 64 lanes of every
+// access to it cover whole consecutive cache lines.  (With 8 fp32 elements a lane, two 16-byte
+// accesses 32 bytes apart, each instruction touched every line half: 69.4 % of the HBM peak on
+// 5.45 GB against 75.5 % this way; the library's plain copy kernel reaches 75.8 %.)  Rows per
+// thread, all loaded before the first use: 4 and 2 -- with 4 elements a lane 1 to 4 rows were
+// timed, 2 is never behind; more rows in flight per thread lose (8: 59 %).
+template <typename TO>
+struct MergeShape {
+  static constexpr int E = sizeof(TO) == 4 ? 4 : 8;
+  static constexpr int ROWS = sizeof(TO) == 4 ? 2 : 4;
+};
+
+// LPR = lanes per row (power of two, LPR * E >= head_dim).
 template <typename TO, typename TN, int LPR>
 __global__ __launch_bounds__(kThreads) void merge_kernel(const MergeArgs a) {
+  constexpr int E = MergeShape<TO>::E;
+  constexpr int kRowsPerThread = MergeShape<TO>::ROWS;
   constexpr int RP = kThreads / LPR;          // rows per pass
   constexpr int BS = RP * kRowsPerThread;     // rows per block
   const int bid = blockIdx.x;
@@ -94,7 +154,7 @@ __global__ __launch_bounds__(kThreads) void merge_kernel(const MergeArgs a) {
   const int st = rest % a.n_stile;
   const int b = rest / a.n_stile;
   const int r = threadIdx.x / LPR;
-  const int c = (threadIdx.x % LPR) * 8;
+  const int c = (threadIdx.x % LPR) * E;
   const bool col_ok = c < a.head_dim;
 
   TO* o = (TO*)a.o + (int64_t)b * a.o_st[0] + (int64_t)h * a.o_st[2] + c;
@@ -102,7 +162,7 @@ __global__ __launch_bounds__(kThreads) void merge_kernel(const MergeArgs a) {
   const int64_t l_base = (int64_t)b * a.l_st[0] + (int64_t)h * a.l_st[1];
   const int64_t ln_base = (int64_t)b * a.ln_st[0] + (int64_t)h * a.ln_st[1];
 
-  float xo[kRowsPerThread][8], xn[kRowsPerThread][8];
+  float xo[kRowsPerThread][E], xn[kRowsPerThread][E];
   float la[kRowsPerThread], lb[kRowsPerThread];
   const int s0 = st * BS + r;
 
@@ -115,8 +175,8 @@ __global__ __launch_bounds__(kThreads) void merge_kernel(const MergeArgs a) {
       lb[i] = a.lsen_f64 ? (float)((const double*)a.lsen)[ln_base + (int64_t)s * a.ln_st[2]]
                          : ((const float*)a.lsen)[ln_base + (int64_t)s * a.ln_st[2]];
       if (col_ok) {
-        Vec8<TO>::load(o + (int64_t)s * a.o_st[1], xo[i]);
-        Vec8<TN>::load(on + (int64_t)s * a.on_st[1], xn[i]);
+        Vec<TO, E>::load(o + (int64_t)s * a.o_st[1], xo[i]);
+        Vec<TN, E>::load(on + (int64_t)s * a.on_st[1], xn[i]);
       }
     }
   }
@@ -133,15 +193,15 @@ __global__ __launch_bounds__(kThreads) void merge_kernel(const MergeArgs a) {
       const float w_old = both_empty ? 0.f : 1.f / (1.f + __expf(diff));
       const float w_new = both_empty ? 0.f : 1.f / (1.f + __expf(-diff));
       if (col_ok) {
-        float y[8];
+        float y[E];
 #pragma unroll
-        for (int j = 0; j < 8; j++) {
+        for (int j = 0; j < E; j++) {
           // a zero weight must annihilate whatever garbage the other side holds
           const float t0 = (w_old == 0.f) ? 0.f : xo[i][j] * w_old;
           const float t1 = (w_new == 0.f) ? 0.f : xn[i][j] * w_new;
           y[j] = t0 + t1;
         }
-        Vec8<TO>::store(o + (int64_t)s * a.o_st[1], y);
+        Vec<TO, E>::store(o + (int64_t)s * a.o_st[1], y);
       }
       if ((threadIdx.x % LPR) == 0) {
         const float m = fmaxf(la[i], lb[i]);
@@ -155,114 +215,16 @@ __global__ __launch_bounds__(kThreads) void merge_kernel(const MergeArgs a) {
   }
 }
 
-#ifdef RSWA_MERGE_E4
-// experiment: 4 elements per lane (every wave instruction fully coalesced), ROWS rows per thread
-template <typename T> struct Vec4;
-template <> struct Vec4<float> {
-  static __device__ __forceinline__ void load(const float* p, float (&x)[4]) {
-    f32x4 a = __builtin_nontemporal_load((const f32x4*)p);
-    for (int i = 0; i < 4; i++) x[i] = a[i];
-  }
-  static __device__ __forceinline__ void store(float* p, const float (&x)[4]) {
-    f32x4 a = {x[0], x[1], x[2], x[3]};
-    __builtin_nontemporal_store(a, (f32x4*)p);
-  }
-};
-template <> struct Vec4<__bf16> {
-  static __device__ __forceinline__ void load(const __bf16* p, float (&x)[4]) {
-    u32x2 a = __builtin_nontemporal_load((const u32x2*)p);
-    for (int i = 0; i < 2; i++) {
-      x[2 * i] = __uint_as_float(a[i] << 16);
-      x[2 * i + 1] = __uint_as_float(a[i] & 0xffff0000u);
-    }
-  }
-  static __device__ __forceinline__ void store(__bf16* p, const float (&x)[4]) {
-    f32x4 f = {x[0], x[1], x[2], x[3]};
-    bf16x4 h = __builtin_convertvector(f, bf16x4);
-    __builtin_nontemporal_store(h, (bf16x4*)p);
-  }
-};
-#ifndef RSWA_MERGE_E4_ROWS
-#define RSWA_MERGE_E4_ROWS 8
-#endif
-template <typename TO, typename TN>
-__global__ __launch_bounds__(kThreads) void merge_kernel_e4(const MergeArgs a) {
-  constexpr int LPR = 32, RP = kThreads / LPR, NR = RSWA_MERGE_E4_ROWS, BS = RP * NR;
-  const int bid = blockIdx.x;
-  const int h = bid % a.heads;
-  const int rest = bid / a.heads;
-  const int st = rest % a.n_stile;
-  const int b = rest / a.n_stile;
-  const int r = threadIdx.x / LPR;
-  const int c = (threadIdx.x % LPR) * 4;
-  TO* o = (TO*)a.o + (int64_t)b * a.o_st[0] + (int64_t)h * a.o_st[2] + c;
-  const TN* on = (const TN*)a.on + (int64_t)b * a.on_st[0] + (int64_t)h * a.on_st[2] + c;
-  const int64_t l_base = (int64_t)b * a.l_st[0] + (int64_t)h * a.l_st[1];
-  const int64_t ln_base = (int64_t)b * a.ln_st[0] + (int64_t)h * a.ln_st[1];
-  float xo[NR][4], xn[NR][4], la[NR], lb[NR];
-  const int s0 = st * BS + r;
-#pragma unroll
-  for (int i = 0; i < NR; i++) {
-    const int s = s0 + i * RP;
-    if (s < a.seqlen) {
-      la[i] = a.lse_f64 ? (float)((const double*)a.lse)[l_base + (int64_t)s * a.l_st[2]]
-                        : ((const float*)a.lse)[l_base + (int64_t)s * a.l_st[2]];
-      lb[i] = a.lsen_f64 ? (float)((const double*)a.lsen)[ln_base + (int64_t)s * a.ln_st[2]]
-                         : ((const float*)a.lsen)[ln_base + (int64_t)s * a.ln_st[2]];
-      Vec4<TO>::load(o + (int64_t)s * a.o_st[1], xo[i]);
-      Vec4<TN>::load(on + (int64_t)s * a.on_st[1], xn[i]);
-    }
-  }
-#pragma unroll
-  for (int i = 0; i < NR; i++) {
-    const int s = s0 + i * RP;
-    if (s < a.seqlen) {
-      const float ninf = -__builtin_inff();
-      const bool both_empty = (la[i] == ninf) && (lb[i] == ninf);
-      const float diff = both_empty ? 0.f : lb[i] - la[i];
-      const float w_old = both_empty ? 0.f : 1.f / (1.f + __expf(diff));
-      const float w_new = both_empty ? 0.f : 1.f / (1.f + __expf(-diff));
-      float y[4];
-#pragma unroll
-      for (int j = 0; j < 4; j++) {
-        const float t0 = (w_old == 0.f) ? 0.f : xo[i][j] * w_old;
-        const float t1 = (w_new == 0.f) ? 0.f : xn[i][j] * w_new;
-        y[j] = t0 + t1;
-      }
-      Vec4<TO>::store(o + (int64_t)s * a.o_st[1], y);
-      if ((threadIdx.x % LPR) == 0) {
-        const float m = fmaxf(la[i], lb[i]);
-        const float merged = both_empty ? ninf : m + log1pf(__expf(-fabsf(diff)));
-        if (a.lse_f64) ((double*)a.lse)[l_base + (int64_t)s * a.l_st[2]] = (double)merged;
-        else ((float*)a.lse)[l_base + (int64_t)s * a.l_st[2]] = merged;
-      }
-    }
-  }
-}
-#endif
-
 template <typename TO, typename TN>
 int launch_merge(const MergeArgs& a, int64_t batch, hipStream_t stream) {
-#ifdef RSWA_MERGE_E4
-  if constexpr ((std::is_same_v<TO, float> || std::is_same_v<TO, __bf16>) && std::is_same_v<TN, __bf16>) {
-    if (a.head_dim == 128) {
-      MergeArgs args = a;
-      constexpr int BS = (kThreads / 32) * RSWA_MERGE_E4_ROWS;
-      args.n_stile = (int)ceil_div(a.seqlen, BS);
-      const int64_t blocks = (int64_t)args.n_stile * a.heads * batch;
-      clear_launch_error();
-      hipLaunchKernelGGL((merge_kernel_e4<TO, TN>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, args);
-      return check_launch("merge_attn_out");
-    }
-  }
-#endif
-  const int chunks = (a.head_dim + 7) / 8;
+  constexpr int E = MergeShape<TO>::E;
+  const int chunks = (a.head_dim + E - 1) / E;
   int lpr = 1;
   while (lpr < chunks) lpr *= 2;
   MergeArgs args = a;
   auto go = [&](auto lpr_c) {
     constexpr int LPR = decltype(lpr_c)::value;
-    constexpr int BS = (kThreads / LPR) * kRowsPerThread;
+    constexpr int BS = (kThreads / LPR) * MergeShape<TO>::ROWS;
     args.n_stile = (int)ceil_div(a.seqlen, BS);
     const int64_t blocks = (int64_t)args.n_stile * a.heads * batch;
     if (blocks == 0) return;
@@ -276,7 +238,8 @@ int launch_merge(const MergeArgs& a, int64_t batch, hipStream_t stream) {
     case 4: go(std::integral_constant<int, 4>{}); break;
     case 8: go(std::integral_constant<int, 8>{}); break;
     case 16: go(std::integral_constant<int, 16>{}); break;
-    default: go(std::integral_constant<int, 32>{}); break;
+    case 32: go(std::integral_constant<int, 32>{}); break;
+    default: go(std::integral_constant<int, 64>{}); break;
   }
   return check_launch("merge_attn_out");
 }

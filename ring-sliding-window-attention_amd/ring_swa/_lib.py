@@ -79,7 +79,11 @@ class AttnParams(Structure):
         ("dk2", c_void_p),
         ("dv2", c_void_p),
         ("ds_handoff", c_int32),
+        ("wide", c_int32),
+        ("dkv_accumulate", c_int32),
     ]
+
+WIDE_OUT, WIDE_DQ, WIDE_DKV = 1, 2, 4
 
 
 class RswaError(RuntimeError):

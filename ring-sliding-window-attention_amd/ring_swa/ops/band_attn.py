@@ -138,6 +138,7 @@ def attn_fwd(
     mask_shift: Optional[int] = None,
     accumulate_into: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
     second: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+    into: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     """Masked attention forward on the HIP kernel; returns ``(out, lse)``.
 
@@ -148,7 +149,13 @@ def attn_fwd(
     ``accumulate_into=(out, lse)``: running partial results of these rows (``out`` in q's
     dtype, ``lse`` fp32, views allowed) that this block is merged into in place, in the
     kernel's epilogue -- the same bits as a forward into temporaries followed by
-    ``merge_attn_out``, without the temporaries and the second pass."""
+    ``merge_attn_out``, without the temporaries and the second pass.  The pair may also be the
+    ring loops' accumulators, ``out`` fp32 and ``lse`` fp64
+    (``ring_swa/sliding_window/nonvarlen.py:53-59``).
+
+    ``into=(out, lse)``: write the block's result into these buffers instead of fresh ones (same
+    two type pairs; as fp32 the values are the block's 16-bit output, exactly) -- how a ring loop
+    starts its accumulators without zero-filling them first."""
     packed = cu_seqlens_q is not None
     _check_qkv(q, k, v, packed)
     assert second is None or k.numel() > 0, "two key ranges: the first must not be empty"
@@ -156,17 +163,24 @@ def attn_fwd(
     if softmax_scale is None:
         softmax_scale = q.shape[-1] ** (-0.5)
     lse_shape = (q.shape[1], q.shape[0]) if packed else (q.shape[0], q.shape[2], q.shape[1])
-    if accumulate_into is not None:
-        out, lse = accumulate_into
-        assert out.shape == q.shape and out.dtype == q.dtype and out.stride(-1) == 1, (
-            "accumulate_into: out must have q's shape and dtype"
+    wide = False
+    assert accumulate_into is None or into is None
+    if accumulate_into is not None or into is not None:
+        out, lse = accumulate_into if accumulate_into is not None else into
+        wide = out.dtype == torch.float32
+        assert out.shape == q.shape and out.stride(-1) == 1 and tuple(lse.shape) == lse_shape, (
+            "out must have q's shape, lse [batch, heads, seq] ([heads, tokens] when packed)"
         )
-        assert tuple(lse.shape) == lse_shape and lse.dtype == torch.float32, (
-            "accumulate_into: lse must be fp32 [batch, heads, seq] ([heads, tokens] when packed)"
+        assert (out.dtype, lse.dtype) in ((q.dtype, torch.float32), (torch.float32, torch.float64)), (
+            "out / lse must be q's dtype / fp32, or the ring accumulators' fp32 / fp64"
         )
         _lib.require_device(out, lse)
-        if q.numel() == 0 or k.numel() == 0:
+        if accumulate_into is not None and (q.numel() == 0 or k.numel() == 0):
             return out, lse  # an empty block is the identity of the merge
+        if into is not None and (q.numel() == 0 or k.numel() == 0):
+            out.zero_()
+            lse.fill_(float("-inf"))
+            return out, lse
     else:
         out = torch.empty(q.shape, dtype=q.dtype, device=dev)
         lse = torch.empty(lse_shape, dtype=torch.float32, device=dev)
@@ -184,6 +198,7 @@ def attn_fwd(
     p.lse = lse.data_ptr()
     p.lse_stride = _lib.i64x3(_lse_strides(lse, packed))
     p.out_accumulate = 0 if accumulate_into is None else 1
+    p.wide = _lib.WIDE_OUT if wide else 0
     with torch.cuda.device(dev):
         _lib.check(_lib.lib().rswa_attn_fwd(p, _lib.stream_ptr(dev)))
     return out, lse
@@ -205,6 +220,7 @@ def attn_bwd(
     static_workspace: bool = False,
     second: Optional[Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]] = None,
     handoff=None,
+    dkv_accumulate: bool = False,
 ) -> None:
     """Masked attention backward; overwrites ``dq, dk, dv`` (views are fine).
 
@@ -219,6 +235,11 @@ def attn_bwd(
     ``static_workspace=True`` runs the whole backward on the library's built-in statistics
     buffer (``rswa_attn_bwd_static``): no device memory is allocated by the call; sizes
     beyond the buffer raise ``NotImplementedError`` and overlapping calls on one GPU race.
+
+    ``dq``, and ``dk`` / ``dv`` together, may also be fp32 -- the ring loops' gradient accumulators
+    (``ring_swa/sliding_window/nonvarlen.py:203-206``): the block's 16-bit gradients are then
+    written as fp32, or with ``dq_accumulate`` / ``dkv_accumulate`` (fp32 ``dk`` / ``dv`` only)
+    added to what the buffers hold, the sums of ``:318-321`` without their elementwise passes.
 
     ``handoff``: dS hand-off (``ds_handoff`` of the ABI) -- the dK/dV kernel stores its 16-bit dS
     tiles in the workspace and dQ comes from a kernel that only multiplies them with K instead
@@ -237,9 +258,10 @@ def attn_bwd(
     assert o.shape == q.shape and do.shape == q.shape and dq.shape == q.shape
     assert dk.shape == k.shape and dv.shape == v.shape
     assert o.dtype == q.dtype and do.dtype == q.dtype
-    assert dq.dtype == q.dtype and dk.dtype == q.dtype and dv.dtype == q.dtype, (
-        "dq, dk, dv must have the dtype of q"
-    )
+    assert dq.dtype in (q.dtype, torch.float32) and dk.dtype in (q.dtype, torch.float32) and \
+        dv.dtype == dk.dtype, "dq and dk / dv must have the dtype of q, or be fp32 accumulators"
+    wide_dq, wide_dkv = dq.dtype == torch.float32, dk.dtype == torch.float32
+    assert not dkv_accumulate or wide_dkv, "dkv_accumulate needs fp32 dk / dv"
     assert softmax_lse.dtype == torch.float32, "softmax_lse must be fp32"
     for t in (o, do, dq, dk, dv):
         assert t.stride(-1) == 1, "last dimension must be contiguous"
@@ -253,7 +275,7 @@ def attn_bwd(
         # nothing to attend: the outputs of the requested phases are zero
         if (phases & 4) and not dq_accumulate:
             dq.zero_()
-        if phases & 2:
+        if (phases & 2) and not dkv_accumulate:
             dk.zero_()
             dv.zero_()
         return
@@ -263,12 +285,14 @@ def attn_bwd(
         dk2, dv2 = second[2], second[3]
         _lib.require_device(dk2, dv2)
         assert dk2.shape == second[0].shape and dv2.shape == second[1].shape
-        assert dk2.dtype == q.dtype and dv2.dtype == q.dtype
+        assert dk2.dtype == dk.dtype and dv2.dtype == dk.dtype
         assert _same_strides(dk2, dk) and _same_strides(dv2, dv), (
             "dk2 / dv2 must have the strides of dk / dv"
         )
         p.dk2, p.dv2 = dk2.data_ptr(), dv2.data_ptr()
     p.dq_accumulate = int(bool(dq_accumulate))
+    p.dkv_accumulate = int(bool(dkv_accumulate))
+    p.wide = (_lib.WIDE_DQ if wide_dq else 0) | (_lib.WIDE_DKV if wide_dkv else 0)
     p.out = o.data_ptr()
     p.out_stride = _lib.i64x3(_strides3(o, packed))
     p.lse = softmax_lse.data_ptr()

@@ -45,7 +45,7 @@ def test_python_struct_matches_c_struct():
 
     L = _lib.lib()
     assert L.rswa_sizeof_attn_params() == ctypes.sizeof(_lib.AttnParams)
-    assert L.rswa_version() == 2
+    assert L.rswa_version() == 3
 
 
 def test_header_cites_reference_interfaces():
