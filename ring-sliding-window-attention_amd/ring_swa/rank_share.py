@@ -21,7 +21,7 @@ from typing import List, Optional, Sequence, Tuple
 import torch
 
 from .ops.accum import (flash_attn_bwd_func, flash_attn_fwd_func, flash_attn_varlen_bwd_func,
-                        flash_attn_varlen_fwd_func)
+                        flash_attn_varlen_fwd_func, hip_kernels)
 from .ops.band_attn import attn_bwd, attn_fwd, bwd_workspace_bytes
 
 Step = Tuple[int, slice, slice, Tuple[int, int], bool]
@@ -148,7 +148,7 @@ class RankShareVarlenFunc(torch.autograd.Function):
         out, lse = _forward_blocks(q4, k4, v4, prev4, plan, softmax_scale, cu_dev, ring_dtypes)
         out, lse = out.squeeze(0), lse.squeeze(0)
         ctx.save_for_backward(q, k, v, out, lse, cu_dev, *prev_kv)
-        ctx.plan, ctx.scale = plan, softmax_scale
+        ctx.plan, ctx.scale, ctx.ring_dtypes = plan, softmax_scale, ring_dtypes
         return out
 
     @staticmethod
@@ -157,7 +157,7 @@ class RankShareVarlenFunc(torch.autograd.Function):
         prev4 = [p.unsqueeze(1) for p in prev_kv]
         grads = _backward_blocks(q.unsqueeze(0), k.unsqueeze(0), v.unsqueeze(0), prev4,
                                  out.unsqueeze(0), lse.unsqueeze(0), do.unsqueeze(0), ctx.plan,
-                                 ctx.scale, cu_dev)
+                                 ctx.scale, cu_dev, ctx.ring_dtypes)
         dprev = [g.squeeze(1) for g in grads[3:]]
         return (grads[0].squeeze(0), grads[1].squeeze(0), grads[2].squeeze(0), None, None, None,
                 None, None, None, *dprev)
@@ -188,25 +188,86 @@ def _join(side: "torch.cuda.Stream", device: torch.device) -> None:
     torch.cuda.current_stream(device).wait_stream(side)
 
 
-def _forward_blocks_accum(q, k, v, prev_kv, plan, scale, local_cu):
-    """The blocks through the accumulating block operators, upstream's flow and accumulator
-    types (``ring_swa/sliding_window/nonvarlen.py:53-59, 95-154``): fp32 output and fp64 LSE
-    start from the merge identity, every block is merged into its row range, one cast at the
-    end."""
+def blocks_forward(q, kv, kv_of, plan, scale, local_cu, kernels=None, before_rest=None):
+    """The planned blocks of one rank through the accumulating block operators -- upstream's flow
+    and accumulator types (``ring_swa/sliding_window/nonvarlen.py:53-59, 95-154``): fp32 output
+    and fp64 LSE, every block merged into its row range; returns the accumulators before their
+    final cast.  ``kv`` is the rank's own stacked chunk ``[2, batch, seq, kv_heads, dim]``,
+    ``kv_of[i]`` the stacked key range the block of step ``i`` reads (of rank ``rank - i``:
+    received by a ring, sliced from a held chunk by the single-GPU emulation), ``local_cu`` the
+    device ``cu_seqlens`` of the own-chunk block of a packed chunk (batch 1).  ``before_rest`` is
+    called between the own-chunk block and the others (a ring waits for its receives there).
+    This one function is what ``ring_rank_share_attn(ring_dtypes=True)``, plans of three and
+    more blocks and the ring over a ``cp_group`` (``ring_swa/ring.py``) all run; on the HIP library
+    the operators work in the kernels' epilogues: the own-chunk block writes the accumulators
+    (they are never filled with the merge identity), the others merge into them, no temporary,
+    no merge launch."""
+    assert plan and plan[0][0] == 0, "the diagonal block comes first: it covers every row"
     b, s, hq, _ = q.shape
-    out = torch.zeros_like(q, dtype=torch.float32)
-    lse = torch.full((b, hq, s), float("-inf"), dtype=torch.float64, device=q.device)
-    for (i, qs, ks, window, causal) in plan:
-        if i == 0:
-            kv = torch.stack([k, v])
-            if local_cu is not None:
-                flash_attn_varlen_fwd_func(q, kv, scale, window, local_cu, local_cu, None, None,
-                                           causal, out, lse)
-            else:
-                flash_attn_fwd_func(q, kv, scale, window, causal, out, lse)
-        else:
-            flash_attn_fwd_func(q[:, qs], prev_kv[i - 1][:, :, ks], scale, window, causal,
-                                out[:, qs], lse[:, :, qs])
+    out = torch.empty(q.shape, dtype=torch.float32, device=q.device)
+    lse = torch.empty((b, hq, s), dtype=torch.float64, device=q.device)
+    (_, _, _, window0, causal0) = plan[0]
+    if local_cu is not None:
+        flash_attn_varlen_fwd_func(q, kv, scale, window0, local_cu, local_cu, None, None, causal0,
+                                   out, lse, kernels=kernels, fresh=True)
+    else:
+        flash_attn_fwd_func(q, kv, scale, window0, causal0, out, lse, kernels=kernels, fresh=True)
+    if before_rest is not None:
+        before_rest()
+    for (i, qs, _, window, causal) in plan[1:]:
+        flash_attn_fwd_func(q[:, qs], kv_of[i], scale, window, causal, out[:, qs], lse[:, :, qs],
+                            kernels=kernels)
+    return out, lse
+
+
+def blocks_backward(q, kv, kv_of, out, lse, do, plan, scale, local_cu, dkv_of, kernels=None,
+                    after_rest=None):
+    """Backward of the same blocks from the final 16-bit ``out`` and fp32 ``lse``
+    (``ring_swa/sliding_window/nonvarlen.py:203-206, 233-321``): returns fp32 ``dq`` and fp32
+    ``dkv`` of the own chunk; the gradients of the key range of step ``i`` are written, in the
+    keys' type, into ``dkv_of[i]`` (a ring sends them back to the keys' owner; the emulation
+    passes views of the held chunks' gradients).  The blocks on other ranks' keys run first and
+    ``after_rest`` is called before the own-chunk block, so that a ring has their gradients on
+    the wire while it computes its largest block.  ``dq`` is never zero-filled: the first block
+    writes its rows (every later block's rows lie inside them: the plans' row ranges are
+    prefixes that shrink with the hop), the rows beyond get zeros, every further block adds."""
+    assert plan and plan[0][0] == 0
+    if len(plan) == 2 and (kernels is None or kernels is hip_kernels()) and q.is_cuda:
+        # exactly one other block, on the HIP library: the two-stream schedule (same sums)
+        i1 = plan[1][0]
+        return _backward_two_blocks(q, kv[0], kv[1], kv_of[i1], dkv_of[i1], out, lse, do, plan,
+                                    scale, local_cu, wide=True, after_rest=after_rest)
+    dq = torch.empty(q.shape, dtype=torch.float32, device=q.device)
+    dkv = torch.empty(kv.shape, dtype=torch.float32, device=q.device)
+    first = True
+    covered = q.shape[1]
+    for (i, qs, _, window, causal) in plan[1:]:
+        q0, q1, _ = qs.indices(q.shape[1])
+        assert q0 == 0 and q1 <= covered, "row ranges of the plan must be shrinking prefixes"
+        if first:
+            dq[:, q1:].zero_()
+            covered = q1
+        flash_attn_bwd_func(q[:, qs], kv_of[i], out[:, qs], lse[:, :, qs], do[:, qs], dq[:, qs],
+                            dkv_of[i], scale, window, causal, kernels=kernels,
+                            accumulate_dq=not first)
+        first = False
+    if after_rest is not None:
+        after_rest()
+    (_, _, _, window0, causal0) = plan[0]
+    if local_cu is not None:
+        flash_attn_varlen_bwd_func(q, kv, out, lse, do, dq, dkv, local_cu, local_cu, None, None,
+                                   scale, window0, causal0, kernels=kernels,
+                                   accumulate_dq=not first)
+    else:
+        flash_attn_bwd_func(q, kv, out, lse, do, dq, dkv, scale, window0, causal0, kernels=kernels,
+                            accumulate_dq=not first)
+    return dq, dkv
+
+
+def _forward_blocks_accum(q, k, v, prev_kv, plan, scale, local_cu):
+    """``blocks_forward`` on key ranges sliced from the held chunks of earlier ranks."""
+    kv_of = {i: prev_kv[i - 1][:, :, ks] for (i, _, ks, _, _) in plan[1:]}
+    out, lse = blocks_forward(q, torch.stack([k, v]), kv_of, plan, scale, local_cu)
     return out.to(q.dtype), lse.float()
 
 
@@ -274,38 +335,37 @@ def _backward_blocks(q, k, v, prev_kv, out, lse, do, plan, scale, local_cu, ring
     if do.stride(-1) != 1:
         do = do.contiguous()
     assert plan and plan[0][0] == 0
-    if len(plan) == 2:
-        one = _one_pass(q, k, v, prev_kv, plan, local_cu) if one_pass and not ring_dtypes else None
+    if len(plan) == 1 and not ring_dtypes:
+        # the own-chunk block alone (rank 0, or a window that ends inside the chunk for a pack
+        # whose first sequence starts in it): 16-bit gradients straight from the kernels
+        dq, dkv = torch.empty_like(q), torch.empty_like(torch.stack([k, v]))
+        (_, _, _, window, causal) = plan[0]
+        if local_cu is not None:
+            flash_attn_varlen_bwd_func(q, torch.stack([k, v]), out, lse, do, dq, dkv, local_cu,
+                                       local_cu, None, None, scale, window, causal)
+        else:
+            flash_attn_bwd_func(q, torch.stack([k, v]), out, lse, do, dq, dkv, scale, window, causal)
+        return (dq, dkv[0], dkv[1], *[torch.zeros_like(kv) for kv in prev_kv])
+    if len(plan) == 2 and not ring_dtypes:
+        one = _one_pass(q, k, v, prev_kv, plan, local_cu) if one_pass else None
         if one is not None:
             return _backward_one_pass(q, k, v, prev_kv, out, lse, do, one, scale)
-        return _backward_two_blocks(q, k, v, prev_kv, out, lse, do, plan, scale, local_cu)
-    # one block, or three and more: the accumulating flow of upstream's backward
-    # (ring_swa/sliding_window/nonvarlen.py:203-206, 233-321) on the block operators; dq and
-    # the own chunk's dkv are summed in fp32, the previous chunks' gradients are what a ring
-    # would send back
-    if len(plan) == 1:
-        dq, dkv = torch.empty_like(q), torch.empty_like(torch.stack([k, v]))
-    else:
-        dq = torch.zeros_like(q, dtype=torch.float32)
-        dkv = torch.empty_like(torch.stack([k, v]))
+        # (the previous chunk's dK / dV are zeroed whole: one contiguous fill is faster than a
+        # strided one of half the size)
+        dprev = [torch.zeros_like(kv) for kv in prev_kv]
+        (i1, _, ks, _, _) = plan[1]
+        dq, dkv = _backward_two_blocks(q, k, v, prev_kv[i1 - 1][:, :, ks], dprev[i1 - 1][:, :, ks],
+                                       out, lse, do, plan, scale, local_cu)
+        return (dq, dkv[0], dkv[1], *dprev)
+    # one block, three and more, or upstream's accumulator types asked for: the accumulating
+    # flow of upstream's backward on the block operators; the previous chunks' gradients are what
+    # a ring would send back (zero outside the key ranges the blocks read)
     dprev = [torch.zeros_like(kv) for kv in prev_kv]
-    for (i, qs, ks, window, causal) in plan:
-        if i == 0:
-            kv = torch.stack([k, v])
-            dq_0 = dq if len(plan) == 1 else torch.empty_like(q)
-            if local_cu is not None:
-                flash_attn_varlen_bwd_func(q, kv, out, lse, do, dq_0, dkv, local_cu, local_cu,
-                                           None, None, scale, window, causal)
-            else:
-                flash_attn_bwd_func(q, kv, out, lse, do, dq_0, dkv, scale, window, causal)
-            if len(plan) > 1:
-                dq += dq_0
-        else:
-            dq_i = torch.empty_like(q[:, qs])
-            flash_attn_bwd_func(q[:, qs], prev_kv[i - 1][:, :, ks], out[:, qs], lse[:, :, qs],
-                                do[:, qs], dq_i, dprev[i - 1][:, :, ks], scale, window, causal)
-            dq[:, qs] += dq_i
-    return (dq.to(q.dtype), dkv[0], dkv[1], *dprev)
+    kv_of = {i: prev_kv[i - 1][:, :, ks] for (i, _, ks, _, _) in plan[1:]}
+    dkv_of = {i: dprev[i - 1][:, :, ks] for (i, _, ks, _, _) in plan[1:]}
+    dq, dkv = blocks_backward(q, torch.stack([k, v]), kv_of, out, lse, do, plan, scale, local_cu,
+                              dkv_of)
+    return (dq.to(q.dtype), dkv[0].to(k.dtype), dkv[1].to(v.dtype), *dprev)
 
 
 def _backward_one_pass(q, k, v, prev_kv, out, lse, do, one, scale):
@@ -330,40 +390,44 @@ def _backward_one_pass(q, k, v, prev_kv, out, lse, do, one, scale):
     return (dq, dk, dv, *dprev)
 
 
-def _backward_two_blocks(q, k, v, prev_kv, out, lse, do, plan, scale, local_cu):
-    """Own-chunk block + one previous-chunk block (window no longer than a chunk): dq is
-    summed inside the dQ kernel instead of in separate passes.  The previous-chunk block
-    writes its dQ first (side stream); the own-chunk dQ kernel, ordered after
-    it, adds to it: fp32 sum of the two 16-bit partials, rounded once -- bit for bit what
-    the fp32 accumulator of ring_swa/sliding_window/nonvarlen.py:203, 318-321 yields for two
-    blocks.
+def _backward_two_blocks(q, k, v, kv1, dkv1, out, lse, do, plan, scale, local_cu, wide=False,
+                         after_rest=None):
+    """Own-chunk block + one block on another rank's key range ``kv1`` (stacked, already sliced;
+    its gradients go to ``dkv1`` in the keys' type), on two streams, with dq summed inside the dQ
+    kernel instead of in separate passes.  The other block writes its dQ first (side stream); the
+    own-chunk dQ kernel, ordered after it, adds to it: fp32 sum of the two 16-bit partials --
+    rounded once into a 16-bit ``dq``, or kept in the fp32 ``dq`` / ``dk`` / ``dv`` of ``wide=True``
+    (the ring loops' accumulators): bit for bit what the fp32 accumulator of
+    ring_swa/sliding_window/nonvarlen.py:203, 318-321 yields for two blocks, either way.
+    ``after_rest`` is called on the side stream once the other block's launches are enqueued
+    there (a ring starts sending its dKV back from that stream).  Returns ``dq`` and the stacked
+    ``dkv`` of the own chunk.
 
     Launch order (measured; each variant below costs 1-6 % of the step): the side stream
-    gets its launches first and runs the previous-chunk dQ kernel before the previous-chunk
-    dK/dV kernel.  The own-chunk dQ kernel then never waits (what it needs is finished long
-    before the own-chunk dK/dV kernel is), and the previous-chunk dK/dV blocks -- few, of
-    very unequal length -- fill the compute units that the short blocks of the own-chunk
-    dK/dV launch and the tail of the own-chunk dQ launch leave idle.  Delaying the side
-    stream's kernels (zero fills on it, own-chunk launches ahead of it) lets the own-chunk
-    dK/dV launch take every compute unit first and loses that packing."""
+    gets its launches first and runs the other block's dQ kernel before its dK/dV kernel.  The
+    own-chunk dQ kernel then never waits (what it needs is finished long before the own-chunk
+    dK/dV kernel is), and the other block's dK/dV blocks -- few, of very unequal length -- fill
+    the compute units that the short blocks of the own-chunk dK/dV launch and the tail of the
+    own-chunk dQ launch leave idle.  Delaying the side stream's kernels (zero fills on it,
+    own-chunk launches ahead of it) lets the own-chunk dK/dV launch take every compute unit
+    first and loses that packing."""
     PREP, DKDV, DQ = 1, 2, 4
     (_, _, _, window0, causal0), (i1, qs, ks, window1, causal1) = plan
-    # Of dq only the rows outside the previous-chunk block are zeroed (the own-chunk dQ kernel
-    # adds to every row; the previous-chunk kernel writes the block's).  The previous chunk's
-    # dK / dV are zeroed whole: one contiguous fill is faster than a strided one of half the size.
+    # Of dq only the rows outside the other block are zeroed (the own-chunk dQ kernel adds to
+    # every row; the other block's kernel writes its own).
     q0, q1, _ = qs.indices(q.shape[1])
-    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    gdt = torch.float32 if wide else q.dtype
+    dq = torch.empty(q.shape, dtype=gdt, device=q.device)
+    dkv = torch.empty((2,) + tuple(k.shape), dtype=gdt, device=q.device)
+    dk, dv = dkv[0], dkv[1]
     dq[:, :q0].zero_()
     dq[:, q1:].zero_()
-    dprev = [torch.zeros_like(kv) for kv in prev_kv]
-    kk, vv, dkv = prev_kv[i1 - 1][0], prev_kv[i1 - 1][1], dprev[i1 - 1]
     if local_cu is not None:
         need = bwd_workspace_bytes(q[0], k[0], local_cu, local_cu)
     else:
         need = bwd_workspace_bytes(q, k)
     ws = torch.empty(need, dtype=torch.uint8, device=q.device)
-    ws_prev = torch.empty(bwd_workspace_bytes(q[:, qs], kk[:, ks]), dtype=torch.uint8,
-                          device=q.device)
+    ws_prev = torch.empty(bwd_workspace_bytes(q[:, qs], kv1[0]), dtype=torch.uint8, device=q.device)
 
     def own(phases, accumulate):
         if local_cu is not None:
@@ -375,8 +439,8 @@ def _backward_two_blocks(q, k, v, prev_kv, out, lse, do, plan, scale, local_cu):
                      phases=phases, dq_accumulate=accumulate)
 
     def prev(phases):
-        attn_bwd(q[:, qs], kk[:, ks], vv[:, ks], out[:, qs], lse[:, :, qs], do[:, qs], dq[:, qs],
-                 dkv[0][:, ks], dkv[1][:, ks], scale, window1, causal1, workspace=ws_prev,
+        attn_bwd(q[:, qs], kv1[0], kv1[1], out[:, qs], lse[:, :, qs], do[:, qs], dq[:, qs],
+                 dkv1[0], dkv1[1], scale, window1, causal1, workspace=ws_prev,
                  phases=phases, dq_accumulate=False)
 
     side = _fork(q.device)
@@ -385,11 +449,13 @@ def _backward_two_blocks(q, k, v, prev_kv, out, lse, do, plan, scale, local_cu):
         dq_prev_done = torch.cuda.Event()
         dq_prev_done.record(side)
         prev(DKDV)
+        if after_rest is not None:
+            after_rest()
     own(PREP | DKDV, False)
     torch.cuda.current_stream(q.device).wait_event(dq_prev_done)
     own(DQ, True)
     _join(side, q.device)
-    return (dq, dk, dv, *dprev)
+    return dq, dkv
 
 
 def ring_rank_share_attn(

@@ -20,9 +20,12 @@ buffers travel the ring backwards.  Here every rank
 Every plan is computed from ``(seq_len, window, cp_size)`` -- and the global ``cu_seqlens`` of
 a pack -- which all ranks know, so a sender needs no message to learn what a receiver wants.
 
-The compute is expressed in the four block operators of ``ops/accum.py`` with upstream's
-accumulator types (fp32 output, fp64 LSE).  ``kernels`` selects the primitives under them:
-the HIP library by default; the CPU test tier passes stand-ins and runs this file over gloo.
+The compute is ``rank_share.blocks_forward`` / ``blocks_backward`` -- the one implementation of
+a rank's blocks on the four block operators of ``ops/accum.py`` with upstream's accumulator
+types (fp32 output, fp64 LSE, fp32 dq / dkv), which ``ring_rank_share_attn(ring_dtypes=True)``
+runs as well; on the HIP library the accumulators are written and added to in the kernels'
+epilogues.  ``kernels`` selects the primitives under the operators: the HIP library by
+default; the CPU test tier passes stand-ins and runs this file over gloo.
 """
 from __future__ import annotations
 
@@ -30,10 +33,10 @@ from typing import List, Optional, Sequence, Tuple
 
 import torch
 
-from .ops.accum import (flash_attn_bwd_func, flash_attn_fwd_func, flash_attn_varlen_bwd_func,
-                        flash_attn_varlen_fwd_func)
+from .ops.band_attn import attn_fwd
 from .ops.p2p import exchange, get_group_local_to_global_rank_map
-from .rank_share import Step, plan_nonvarlen, plan_varlen, ring_comm_times
+from .rank_share import (Step, _backward_two_blocks, blocks_backward, blocks_forward,
+                         plan_nonvarlen, plan_varlen, ring_comm_times)
 
 
 def _steps_of(rank: int, seq_len: int, window_size: int, cp_size: int,
@@ -57,12 +60,21 @@ def _incoming(rank: int, seq_len: int, window_size: int, cp_size: int, cu_host):
     return out
 
 
-def band_forward(q, kv, window_size, cp_group, cp_size, rank, softmax_scale, kernels, cu_host):
+def band_forward(q, kv, window_size, cp_group, cp_size, rank, softmax_scale, kernels, cu_host,
+                 narrow=False):
     """Forward of the band blocks of one rank on ``[batch, seq, heads, dim]`` chunks (batch 1
     around a packed chunk): returns the accumulators of
     ``ring_swa/sliding_window/nonvarlen.py:53-59`` -- fp32 output, fp64 LSE -- before their
     final cast, the device ``cu_seqlens`` of the own-chunk block (packed), the block plan and
-    the received key ranges by hop."""
+    the received key ranges by hop.
+
+    ``narrow=True`` (HIP library only) lets a plan of exactly two blocks -- the window no longer
+    than a chunk, the common case -- run without the wide accumulators: the second block is merged
+    into the first one's 16-bit output and fp32 LSE in its kernel's epilogue.  One merge, one
+    rounding: the bits the fp32 / fp64 accumulators give after their final cast, without their
+    extra passes over the output (the same two routes of the single-GPU emulation of a rank's
+    step take 2.33 and 2.15 ms per forward + backward at 8192-token chunks, window 4096, 32 / 8
+    heads)."""
     b, s, hq, d = q.shape
     local_cu, steps = _steps_of(rank, s, window_size, cp_size, cu_host)
     cu_dev = None
@@ -81,57 +93,58 @@ def band_forward(q, kv, window_size, cp_group, cp_size, rank, softmax_scale, ker
              for (_, other, ks) in _incoming(rank, s, window_size, cp_size, cu_host)]
     reqs = exchange(sends, recvs, cp_group)
 
-    out = torch.zeros_like(q, dtype=torch.float32)
-    lse = torch.full((b, hq, s), float("-inf"), dtype=torch.float64, device=q.device)
-    (_, _, _, window0, causal0) = steps[0]
-    if cu_host is not None:
-        flash_attn_varlen_fwd_func(q, kv, softmax_scale, window0, cu_dev, cu_dev, None, None,
-                                   causal0, out, lse, kernels=kernels)
-    else:
-        flash_attn_fwd_func(q, kv, softmax_scale, window0, causal0, out, lse, kernels=kernels)
-    for req in reqs:
-        req.wait()
-    for (i, qs, _, window, causal) in steps[1:]:
-        flash_attn_fwd_func(q[:, qs], got[i], softmax_scale, window, causal, out[:, qs],
-                            lse[:, :, qs], kernels=kernels)
+    def landed():
+        for req in reqs:
+            req.wait()
+
+    # own-chunk block while the key ranges are on the wire, then the blocks on them
+    if narrow and kernels is None and len(steps) == 2:
+        (_, _, _, window0, causal0), (i1, qs, _, window1, causal1) = steps
+        if cu_dev is not None:
+            out, lse = attn_fwd(q[0], kv[0][0], kv[1][0], softmax_scale, window0, causal0, cu_dev, cu_dev)
+            out, lse = out.unsqueeze(0), lse.unsqueeze(0)
+        else:
+            out, lse = attn_fwd(q, kv[0], kv[1], softmax_scale, window0, causal0)
+        landed()
+        attn_fwd(q[:, qs], got[i1][0], got[i1][1], softmax_scale, window1, causal1,
+                 accumulate_into=(out[:, qs], lse[:, :, qs]))
+        return out, lse, cu_dev, steps, got
+    out, lse = blocks_forward(q, kv, got, steps, softmax_scale, cu_dev, kernels, before_rest=landed)
     return out, lse, cu_dev, steps, got
 
 
 def band_backward(q, kv, out, lse, do, got_list, window_size, cp_group, cp_size, rank,
-                  softmax_scale, kernels, cu_host, steps, cu_dev):
+                  softmax_scale, kernels, cu_host, steps, cu_dev, narrow=False):
     """Backward of the same blocks from the final ``(out, lse)``: fp32 ``dq`` and ``dkv`` of this
-    rank's chunk, the contributions of later ranks included."""
+    rank's chunk, the contributions of later ranks included.  ``narrow=True``: a plan of two
+    blocks on the HIP library sums its two dq partials inside the dQ kernel and returns 16-bit
+    ``dq``; ``dkv`` is 16-bit unless later ranks contribute to it (then fp32: own gradients and
+    contributions summed in fp32, in hop order, as with the wide accumulators)."""
     s = q.shape[1]
     gmap = get_group_local_to_global_rank_map(cp_group)
-    dq = torch.zeros_like(q, dtype=torch.float32)
-    dkv = torch.zeros_like(kv, dtype=torch.float32)
-
-    # blocks on received key ranges first: their dKV goes back to the owners while the
-    # own-chunk block runs
-    sends = []
-    for (i, qs, _, window, causal), kv_i in zip(steps[1:], got_list):
-        dq_i = torch.empty_like(q[:, qs])
-        dkv_i = torch.empty_like(kv_i)
-        flash_attn_bwd_func(q[:, qs], kv_i, out[:, qs], lse[:, :, qs], do[:, qs], dq_i, dkv_i,
-                            softmax_scale, window, causal, kernels=kernels)
-        dq[:, qs] += dq_i
-        sends.append((dkv_i, gmap[rank - i]))
+    kv_of = {i: kv_i for (i, *_r), kv_i in zip(steps[1:], got_list)}
+    dkv_of = {i: torch.empty_like(kv_i) for i, kv_i in kv_of.items()}
     incoming = _incoming(rank, s, window_size, cp_size, cu_host)
     back = [kv.new_empty((2, kv.shape[1], ks.stop - ks.start, kv.shape[3], kv.shape[4]))
             for (_, _, ks) in incoming]
-    recvs = [(buf, gmap[other]) for buf, (_, other, _) in zip(back, incoming)]
-    reqs = exchange(sends, recvs, cp_group)
+    reqs = []
 
-    (_, _, _, window0, causal0) = steps[0]
-    dq_0, dkv_0 = torch.empty_like(q), torch.empty_like(kv)
-    if cu_host is not None:
-        flash_attn_varlen_bwd_func(q, kv, out, lse, do, dq_0, dkv_0, cu_dev, cu_dev, None, None,
-                                   softmax_scale, window0, causal0, kernels=kernels)
+    def send_back():
+        # the blocks on received key ranges are done: their dKV goes back to the owners while
+        # the own-chunk block runs
+        sends = [(dkv_of[i], gmap[rank - i]) for (i, *_r) in steps[1:]]
+        recvs = [(buf, gmap[other]) for buf, (_, other, _) in zip(back, incoming)]
+        reqs.extend(exchange(sends, recvs, cp_group))
+
+    if narrow and kernels is None and len(steps) == 2:
+        i1 = steps[1][0]
+        dq, dkv = _backward_two_blocks(q, kv[0], kv[1], kv_of[i1], dkv_of[i1], out, lse, do, steps,
+                                       softmax_scale, cu_dev, wide=False, after_rest=send_back)
+        if incoming:
+            dkv = dkv.float()
     else:
-        flash_attn_bwd_func(q, kv, out, lse, do, dq_0, dkv_0, softmax_scale, window0, causal0,
-                            kernels=kernels)
-    dq += dq_0
-    dkv += dkv_0
+        dq, dkv = blocks_backward(q, kv, kv_of, out, lse, do, steps, softmax_scale, cu_dev, dkv_of,
+                                  kernels, after_rest=send_back)
     for req in reqs:
         req.wait()
     for buf, (_, _, ks) in zip(back, incoming):  # hop order: a fixed order of the fp32 sums
@@ -153,7 +166,7 @@ class RingSlidingWindowFunc(torch.autograd.Function):
             softmax_scale = q.shape[-1] ** (-0.5)
         kv = torch.stack([k, v], dim=0)
         out, lse, cu_dev, steps, got = band_forward(q, kv, window_size, cp_group, cp_size, rank,
-                                                    softmax_scale, kernels, cu_host)
+                                                    softmax_scale, kernels, cu_host, narrow=True)
         out = out.to(q.dtype)
         lse = lse.to(torch.float32)
         ctx.save_for_backward(q, kv, out, lse, *(got[i] for (i, *_rest) in steps[1:]))
@@ -171,7 +184,8 @@ class RingSlidingWindowFunc(torch.autograd.Function):
         if do.stride(-1) != 1:
             do = do.contiguous()
         dq, dkv = band_backward(q, kv, out, lse, do, got_list, window_size, cp_group, cp_size,
-                                rank, softmax_scale, kernels, cu_host, steps, ctx.cu_dev)
+                                rank, softmax_scale, kernels, cu_host, steps, ctx.cu_dev,
+                                narrow=True)
         dq, dk, dv = dq.to(q.dtype), dkv[0].to(kv.dtype), dkv[1].to(kv.dtype)
         if packed:
             dq, dk, dv = dq.squeeze(0), dk.squeeze(0), dv.squeeze(0)
