@@ -31,8 +31,8 @@ PEAK_HBM_GBPS = 8000.0     # MI355X HBM3E
 # from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --pmc-pass`, each counter
 # scaled by what it reads for the 1 GiB device copy of that pass (FETCH_SIZE x2.0, WRITE_SIZE
 # x1.0); the summary is profiles/c3_step_kernels_hbm_traffic_pmc.txt.
-DKDV_HBM_BYTES_PER_LAUNCH = 755.9e6
-MERGE_HBM_BYTES_PER_LAUNCH = 5688.8e6
+DKDV_HBM_BYTES_PER_LAUNCH = 748.2e6
+MERGE_HBM_BYTES_PER_LAUNCH = 5452.6e6
 # Untimed steps before the W warm-up steps: an idle GPU takes some tens of milliseconds of load to
 # settle its clocks (the first launches of a run take up to a third longer than the later ones), and
 # W = 5 steps are 10 ms.
@@ -336,6 +336,10 @@ def main():
                 o_b, lse_b = attn_fwd(qd, tk, tv, None, (W, 0), True, second=(kd, vd))
                 attn_bwd(qd, tk, tv, o_b, lse_b, do, dq, dtk, dtv, None, (W, 0), True,
                          second=(kd, vd, dk, dv))
+                # the same backward on the dS hand-off route (dK/dV kernel <..., 1> stores its
+                # dS tiles, attn_bwd_dq_ds_kernel reads them)
+                attn_bwd(qd, tk, tv, o_b, lse_b, do, dq, dtk, dtv, None, (W, 0), True,
+                         second=(kd, vd, dk, dv), handoff=True)
             torch.cuda.synchronize()
         print(json.dumps({"pmc_pass": "done", "copy_bytes_each_way": 1 << 30}))
         return
@@ -475,6 +479,22 @@ def main():
                 "bwd_own_chunk_all_kernels": {"ms": bwd_med, "TFLOP/s": tf(10 * fl_pair, bwd_med),
                                               "flops_per_pair": "10 D (window-effective)"},
             }
+            # the band's backward on the dS hand-off route, beside the recomputing one above
+            ws_h = torch.empty(bwd_workspace_bytes(qd, tk, second_rows=S, window_size=(W, 0), causal=True,
+                                                   handoff=True), dtype=torch.uint8, device=dev)
+            hand = lambda ph: attn_bwd(qd, tk, tv, o_b, lse_b, do, dq, dtk, dtv, None, (W, 0), True,  # noqa: E731
+                                       workspace=ws_h, phases=ph, second=(kd, vd, dk, dv), handoff=True)
+            hand(7)
+            h_dkdv, _ = event_ms(lambda: hand(DKDV), 20)
+            h_dq, _ = event_ms(lambda: hand(DQ), 20)
+            h_all, _ = event_ms(lambda: hand(7), 20)
+            r_all, _ = event_ms(lambda: band(7), 20)
+            rec["kernels"]["bwd_step_band_ds_handoff"] = {
+                "dkdv_ms": h_dkdv, "dq_ms": h_dq, "all_kernels_ms": h_all,
+                "recompute_all_kernels_ms": r_all, "ds_bytes": ws_h.numel() - ws_b.numel(),
+                "note": "opt-in route: the dK/dV kernel stores its 16-bit dS tiles (2 bytes per pair "
+                        "and head), the dQ kernel only multiplies them with K"}
+            del ws_h
             # The dK/dV launch of the own-chunk block alone leaves a quarter of the compute
             # units idle in its tail (256 blocks of unequal length on 256 units); in the
             # two-block form of the rank step the previous-chunk dK/dV launch of the second

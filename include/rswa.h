@@ -21,10 +21,19 @@
  *                         ring_swa/sliding_window/varlen.py:406-417
  *   rswa_attn_bwd         ring_swa/ops/wrap_flash.py:276-327 (wrapped_flash_attn_bwd)
  *                         and :330-429 (wrapped_flash_attn_bwd_varlen)
- *   rswa_attn_bwd_static  (no upstream counterpart: rswa_attn_bwd for callers that
- *                         cannot allocate; see its declaration)
- *   rswa_attn_bwd_workspace_bytes   (sizing helper for the scratch rswa_attn_bwd
- *                         needs; upstream flash-attn allocates the same internally)
+ *   rswa_attn_bwd_phases  the same interface, one launch of the three at a time
+ *   rswa_attn_bwd_static, rswa_attn_bwd_static_init  (no upstream counterpart:
+ *                         rswa_attn_bwd for callers that cannot allocate; see their
+ *                         declarations)
+ *   rswa_attn_bwd_workspace_bytes, rswa_attn_bwd_handoff_active   (sizing helper for the
+ *                         scratch rswa_attn_bwd needs -- upstream flash-attn allocates the
+ *                         same internally -- and which route a backward call takes)
+ *   rswa_stream_copy      (no upstream counterpart: the copy kernel the merge kernel's
+ *                         rate is measured against)
+ * The accumulating forms of the block operators, ring_swa/ops/attn.py:12-196 with the
+ * fp32 / fp64 / fp32 accumulators of ring_swa/sliding_window/nonvarlen.py:53-59, 203-206,
+ * are served by the fields out_accumulate, dq_accumulate, wide and dkv_accumulate of
+ * rswa_attn_params.
  */
 #ifndef RSWA_H
 #define RSWA_H

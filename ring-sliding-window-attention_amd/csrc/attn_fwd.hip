@@ -457,6 +457,8 @@ int launch_fwd(AttnArgs& a, hipStream_t stream) {
   // keys a row sees at most; the per-wave tile skip pays when the rows of a block beyond one
   // wave's 32 add a tenth or more to that span
   const int64_t span = (a.wl < 0 || a.wr < 0) ? (int64_t)1 << 40 : (int64_t)a.wl + a.wr + 1;
+  // (measured at window 1000 and 128-row blocks, where the skip would save a wave one tile in
+  // eighteen: no difference either way, 0.435 against 0.431-0.441 ms)
   const bool skip = (bm - 32) * 10 >= span + bm;
   clear_launch_error();
   const dim3 grid(padded_grid(a.n_work)), block(C::THREADS);

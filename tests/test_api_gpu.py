@@ -160,6 +160,28 @@ def test_rank_shares_concatenate_to_the_global_result(w, cp, ring_dtypes):
     assert (torch.cat(outs, 1) - glob).abs().max().item() <= OUT_TOL
 
 
+@pytest.mark.parametrize("w,s_loc,batch", [(300, 512, 1), (512, 512, 2), (100, 768, 1)])
+def test_two_block_step_is_the_same_bits_with_16_bit_and_with_fp32_accumulators(w, s_loc, batch):
+    """A step of two blocks (window no longer than a chunk): the 16-bit route (second block
+    merged in its forward epilogue, dq summed inside the own-chunk dQ kernel) and the route
+    through the fp32 / fp64 / fp32 accumulators of ring_swa/sliding_window/nonvarlen.py:53-59,
+    203-206 both make one fp32 combination of the two blocks' 16-bit results and round once."""
+    import ring_swa
+
+    hq, hk, d, cp, rank = 8, 2, 128, 4, 2
+    q, do = _rand((batch, s_loc, hq, d), 11), _rand((batch, s_loc, hq, d), 12)
+    k, v = _rand((batch, s_loc, hk, d), 13), _rand((batch, s_loc, hk, d), 14)
+    prev = _rand((2, batch, s_loc, hk, d), 15)
+    got = {}
+    for route, kw in (("narrow", {"one_pass": False}), ("wide", {"ring_dtypes": True})):
+        qg, kg, vg, pg = (t.cuda().requires_grad_() for t in (q, k, v, prev))
+        out = ring_swa.ring_rank_share_attn(qg, kg, vg, [pg], w, cp, rank, **kw)
+        out.backward(do.cuda())
+        got[route] = (out.detach(), qg.grad, kg.grad, vg.grad, pg.grad)
+    for a, b in zip(got["narrow"], got["wide"]):
+        assert a.dtype == b.dtype and torch.equal(a, b)
+
+
 @pytest.mark.parametrize("w", [200, 600])
 def test_rank_shares_varlen_concatenate_to_the_global_result(w):
     import ring_swa
