@@ -163,7 +163,7 @@ class RankShareVarlenFunc(torch.autograd.Function):
                 None, None, None, *dprev)
 
 
-_SIDE_STREAMS = {}
+_SIDE_STREAMS = threading.local()  # .by_device: {device index: stream}; gone with its thread
 
 
 def _fork(device: torch.device) -> "torch.cuda.Stream":
@@ -176,10 +176,12 @@ def _fork(device: torch.device) -> "torch.cuda.Stream":
     orders the caller's stream after them again.  Tensors used on the side stream are
     allocated on the caller's stream before the fork (or marked with ``record_stream``), so
     the caching allocator hands their memory back to the caller's stream only."""
-    key = (device.index, threading.get_ident())
-    side = _SIDE_STREAMS.get(key)
+    by_device = getattr(_SIDE_STREAMS, "by_device", None)
+    if by_device is None:
+        by_device = _SIDE_STREAMS.by_device = {}
+    side = by_device.get(device.index)
     if side is None:
-        side = _SIDE_STREAMS[key] = torch.cuda.Stream(device)
+        side = by_device[device.index] = torch.cuda.Stream(device)
     side.wait_stream(torch.cuda.current_stream(device))
     return side
 
