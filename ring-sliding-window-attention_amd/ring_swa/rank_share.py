@@ -22,7 +22,7 @@ import torch
 
 from .ops.accum import (flash_attn_bwd_func, flash_attn_fwd_func, flash_attn_varlen_bwd_func,
                         flash_attn_varlen_fwd_func, hip_kernels)
-from .ops.band_attn import attn_bwd, attn_fwd, bwd_workspace_bytes
+from .ops.band_attn import attn_bwd, attn_fwd, bwd_handoff_active, bwd_workspace_bytes
 
 Step = Tuple[int, slice, slice, Tuple[int, int], bool]
 
@@ -385,8 +385,12 @@ def _backward_one_pass(q, k, v, prev_kv, out, lse, do, one, scale):
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     dprev = [torch.zeros_like(kv) for kv in prev_kv]
     dkk, dvv = dprev[0][0][:, s - tail:], dprev[0][1][:, s - tail:]
-    ws = torch.empty(bwd_workspace_bytes(q, kk, second_rows=s), dtype=torch.uint8, device=q.device)
-    for phases in (PREP, DQ, DKDV):
+    # (sized for the route attn_bwd will pick: handoff=None on both sides)
+    ws = torch.empty(bwd_workspace_bytes(q, kk, second_rows=s, window_size=(w, 0), causal=True,
+                                         handoff=None), dtype=torch.uint8, device=q.device)
+    handed = bwd_handoff_active(q, kk, second_rows=s, window_size=(w, 0), causal=True)
+    # the dQ kernel of the hand-off route reads what the dK/dV kernel stored
+    for phases in ((PREP, DKDV, DQ) if handed else (PREP, DQ, DKDV)):
         attn_bwd(q, kk, vv, out, lse, do, dq, dkk, dvv, scale, (w, 0), True, workspace=ws,
                  phases=phases, second=(k, v, dk, dv))
     return (dq, dk, dv, *dprev)
@@ -424,6 +428,7 @@ def _backward_two_blocks(q, k, v, kv1, dkv1, out, lse, do, plan, scale, local_cu
     dk, dv = dkv[0], dkv[1]
     dq[:, :q0].zero_()
     dq[:, q1:].zero_()
+    # (the launches below run dQ ahead of dK/dV, which the dS hand-off cannot: handoff=False)
     if local_cu is not None:
         need = bwd_workspace_bytes(q[0], k[0], local_cu, local_cu)
     else:
@@ -435,15 +440,15 @@ def _backward_two_blocks(q, k, v, kv1, dkv1, out, lse, do, plan, scale, local_cu
         if local_cu is not None:
             attn_bwd(q[0], k[0], v[0], out[0], lse[0], do[0], dq[0], dk[0], dv[0], scale, window0,
                      causal0, local_cu, local_cu, workspace=ws, phases=phases,
-                     dq_accumulate=accumulate)
+                     dq_accumulate=accumulate, handoff=False)
         else:
             attn_bwd(q, k, v, out, lse, do, dq, dk, dv, scale, window0, causal0, workspace=ws,
-                     phases=phases, dq_accumulate=accumulate)
+                     phases=phases, dq_accumulate=accumulate, handoff=False)
 
     def prev(phases):
         attn_bwd(q[:, qs], kv1[0], kv1[1], out[:, qs], lse[:, :, qs], do[:, qs], dq[:, qs],
                  dkv1[0], dkv1[1], scale, window1, causal1, workspace=ws_prev,
-                 phases=phases, dq_accumulate=False)
+                 phases=phases, dq_accumulate=False, handoff=False)
 
     side = _fork(q.device)
     with torch.cuda.stream(side):

@@ -114,6 +114,45 @@ def test_config3_rank_share_chunk8192_gqa_window4096(route):
         assert torch.isfinite(t.float()).all()
 
 
+def test_config3_rank_share_on_the_ds_handoff_route(monkeypatch):
+    """The same step with the backward's dS hand-off switched on (RSWA_DS_HANDOFF=1: the dK/dV
+    kernel stores its 16-bit dS tiles, 2.4 GB here, and the dQ kernel multiplies them with K
+    instead of recomputing S and dP; the interface is that of ring_swa/ops/wrap_flash.py:276-327):
+    against the oracle, and against the recomputing route -- dK / dV the same bits, dQ to the
+    rounding of another summation order."""
+    import ring_swa
+    from ring_swa.ops.band_attn import bwd_handoff_active
+
+    s, hq, hk, w, cp, rank = 8192, 32, 8, 4096, 8, 1
+    q, do = _randn((1, s, hq, D), 0), _randn((1, s, hq, D), 1)
+    k, v = _randn((1, s, hk, D), 2), _randn((1, s, hk, D), 3)
+    prev = _randn((2, 1, s, hk, D), 4)
+
+    def step():
+        qg, kg, vg, pg = (t.clone().requires_grad_() for t in (q, k, v, prev))
+        out = ring_swa.ring_rank_share_attn(qg, kg, vg, [pg], w, cp, rank)
+        out.backward(do)
+        return out.detach(), qg.grad, kg.grad, vg.grad, pg.grad
+
+    plain = step()
+    monkeypatch.setenv("RSWA_DS_HANDOFF", "1")
+    assert bwd_handoff_active(q, prev[0][:, s - w:], second_rows=s, window_size=(w, 0), causal=True)
+    out, dq, dk, dv, dprev = step()
+    monkeypatch.delenv("RSWA_DS_HANDOFF")
+    assert torch.equal(out, plain[0])
+    assert torch.equal(dk, plain[2]) and torch.equal(dv, plain[3]) and torch.equal(dprev, plain[4])
+    assert _rel(dq, plain[1]) <= 2e-3
+    gq, gk = slice(0, hq // hk), slice(0, 1)
+    kc = torch.cat([prev[0][:, :, gk], k[:, :, gk]], 1)
+    vc = torch.cat([prev[1][:, :, gk], v[:, :, gk]], 1)
+    ro, _, rq, rk, rv = O.attention_fwd_bwd(
+        lambda q, k, v: O.window_attention(q, k, v, None, (w, 0), True), q[:, :, gq], kc, vc,
+        do[:, :, gq])
+    _check("c3 hand-off", out[:, :, gq], (dq[:, :, gq], dk[:, :, gk], dv[:, :, gk]),
+           ro, (rq, rk[:, s:], rv[:, s:]))
+    assert torch.isfinite(dq.float()).all()
+
+
 def _log_uniform_lengths(total, lo, hi, seed):
     g = torch.Generator().manual_seed(seed)
     lens = []
