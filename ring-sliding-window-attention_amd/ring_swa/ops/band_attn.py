@@ -250,7 +250,8 @@ def attn_bwd(
     tiles the dK/dV kernel splits over several blocks -- ``"force"`` prefers the hand-off to that
     split); ``False`` never.  With
     ``phases`` spread over several calls the same value must be passed to each, on the same
-    workspace, and the dK/dV phase must run before the dQ phase."""
+    workspace, and the dK/dV phase must run before the dQ phase.  A ``workspace`` the caller
+    supplies without room for the dS tiles makes the automatic choice (``None``) recompute."""
     packed = cu_seqlens_q is not None
     _check_qkv(q, k, v, packed)
     assert second is None or k.numel() > 0, "two key ranges: the first must not be empty"
@@ -311,9 +312,17 @@ def attn_bwd(
         return
     _set_handoff(p, handoff)
     need = int(L.rswa_attn_bwd_workspace_bytes(p))
+    if workspace is not None and handoff is None and p.ds_handoff and workspace.numel() < need:
+        # a caller's workspace without room for the dS tiles: the automatic choice recomputes
+        p.ds_handoff = 0
+        need = int(L.rswa_attn_bwd_workspace_bytes(p))
     if workspace is None:
         workspace = torch.empty(need, dtype=torch.uint8, device=dev)  # 512-B aligned by torch
-    assert workspace.dtype == torch.uint8 and workspace.numel() >= need and workspace.device == dev
+    assert workspace.dtype == torch.uint8 and workspace.device == dev
+    assert workspace.numel() >= need, (
+        f"workspace of {workspace.numel()} bytes, {need} needed: size it with bwd_workspace_bytes "
+        "and the mask / num_sink / handoff of this call"
+    )
     p.workspace = workspace.data_ptr()
     p.workspace_bytes = workspace.numel()
     with torch.cuda.device(dev):

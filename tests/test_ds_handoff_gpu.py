@@ -191,3 +191,32 @@ def test_handoff_dq_accumulate_and_stale_workspace():
         attn_bwd(q, k, v, out, lse, do, pq, pk, pv, None, (w, 0), True, workspace=ws, phases=ph,
                  handoff="force")
     assert torch.equal(pq, gq) and torch.equal(pk, gk) and torch.equal(pv, gv)
+
+
+def test_automatic_choice_follows_the_workspace_it_is_given(monkeypatch):
+    """With the route switched on by the environment, a call that brings its own workspace takes
+    the hand-off only if the dS tiles fit in it; sized without them, the call recomputes (same
+    bits as with the route off) instead of failing."""
+    from ring_swa.ops import attn_fwd
+    from ring_swa.ops.band_attn import attn_bwd, bwd_workspace_bytes
+
+    b, s, hq, hk, d, w = 1, 70000, 8, 8, 128, 300   # 274 key blocks x 8 heads: no split launch
+    q, do = _rand((b, s, hq, d), torch.bfloat16, 1).cuda(), _rand((b, s, hq, d), torch.bfloat16, 4).cuda()
+    k, v = _rand((b, s, hk, d), torch.bfloat16, 2).cuda(), _rand((b, s, hk, d), torch.bfloat16, 3).cuda()
+    out, lse = attn_fwd(q, k, v, None, (w, 0), True)
+    ref = [torch.empty_like(t) for t in (q, k, v)]
+    attn_bwd(q, k, v, out, lse, do, *ref, None, (w, 0), True, handoff=False)
+    monkeypatch.setenv("RSWA_DS_HANDOFF", "1")
+    small = bwd_workspace_bytes(q, k, window_size=(w, 0), causal=True, handoff=False)
+    large = bwd_workspace_bytes(q, k, window_size=(w, 0), causal=True, handoff=None)
+    assert large > small
+    got = [torch.empty_like(t) for t in (q, k, v)]
+    attn_bwd(q, k, v, out, lse, do, *got, None, (w, 0), True,
+             workspace=torch.empty(small, dtype=torch.uint8, device="cuda"))
+    assert all(torch.equal(a, b) for a, b in zip(got, ref))
+    handed = [torch.empty_like(t) for t in (q, k, v)]
+    attn_bwd(q, k, v, out, lse, do, *handed, None, (w, 0), True,
+             workspace=torch.empty(large, dtype=torch.uint8, device="cuda"))
+    assert torch.equal(handed[1], ref[1]) and torch.equal(handed[2], ref[2])
+    assert not torch.equal(handed[0], ref[0])  # another summation order: the route was taken
+    assert ((handed[0].float() - ref[0].float()).norm() / ref[0].float().norm()).item() < 2e-3
