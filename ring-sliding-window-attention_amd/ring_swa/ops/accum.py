@@ -5,7 +5,8 @@ Names, positional order and in-place behaviour of the four operators of the upst
 (``ring_swa/ops/attn.py:12-60, 63-126, 129-160, 163-196``), so a ring loop written against
 them runs on this package unchanged:
 
-* ``kv`` is the stacked pair ``[2, batch, seq, kv_heads, dim]``;
+* ``kv`` is the stacked pair ``[2, batch, seq, kv_heads, dim]`` (a caller that holds ``k`` and
+  ``v`` separately may pass the tuple ``(k, v)`` and save the copy);
 * forward: the block's ``(out, lse)`` is merged into ``global_attn_out`` (fp32 upstream) and
   ``global_softmax_lse`` (fp64 upstream, ``[batch, heads, seq]``) in place, whose start
   state ``(0, -inf)`` is the merge identity; sliced views (``[:, :v]``) are fine;
@@ -135,7 +136,7 @@ def flash_attn_fwd_func(
 ) -> None:
     """Dense block forward merged into the accumulators (``ops/attn.py:12-60``)."""
     K = kernels or hip_kernels()
-    sq, sk = q.shape[1], kv.shape[2]
+    sq, sk = q.shape[1], kv[0].shape[1]
     if _one_call(sq, sk, window_size, causal):
         _fwd_into(K, q, kv[0], kv[1], softmax_scale, window_size, causal, None, None,
                   global_attn_out, global_softmax_lse, fresh)
@@ -169,13 +170,13 @@ def flash_attn_bwd_func(
     ``softmax_lse`` views are passed as they are (the kernels take strides; upstream clones
     them, ``:99-101``)."""
     K = kernels or hip_kernels()
-    sq, sk = q.shape[1], kv.shape[2]
+    sq, sk = q.shape[1], kv[0].shape[1]
     if _one_call(sq, sk, window_size, causal):
         _bwd_into(K, q, kv[0], kv[1], o, softmax_lse, do, dq, dkv[0], dkv[1], softmax_scale,
                   window_size, causal, None, None, accumulate_dq, accumulate_dkv)
         return
     # two parts; dkv of the two summed in fp32 and rounded once, as upstream does (:93-126)
-    parts = torch.zeros_like(kv, dtype=torch.float32)
+    parts = torch.zeros((2,) + tuple(kv[0].shape), dtype=torch.float32, device=q.device)
     flash_attn_bwd_func(q[:, :-sk], kv, o[:, :-sk], softmax_lse[:, :, :-sk], do[:, :-sk],
                         dq[:, :-sk], parts, softmax_scale, (-1, -1), causal, kernels=K,
                         accumulate_dq=accumulate_dq, accumulate_dkv=True)
@@ -183,7 +184,7 @@ def flash_attn_bwd_func(
                         dq[:, -sk:], parts, softmax_scale, window_size, causal, kernels=K,
                         accumulate_dq=accumulate_dq, accumulate_dkv=True)
     if accumulate_dkv:
-        dkv += parts.to(kv.dtype)  # (the 16-bit block gradient, then the accumulator's sum)
+        dkv += parts.to(kv[0].dtype)  # (the 16-bit block gradient, then the accumulator's sum)
     else:
         dkv.copy_(parts)
 

@@ -194,7 +194,7 @@ def blocks_forward(q, kv, kv_of, plan, scale, local_cu, kernels=None, before_res
     """The planned blocks of one rank through the accumulating block operators -- upstream's flow
     and accumulator types (``ring_swa/sliding_window/nonvarlen.py:53-59, 95-154``): fp32 output
     and fp64 LSE, every block merged into its row range; returns the accumulators before their
-    final cast.  ``kv`` is the rank's own stacked chunk ``[2, batch, seq, kv_heads, dim]``,
+    final cast.  ``kv`` is the rank's own chunk, stacked ``[2, batch, seq, kv_heads, dim]`` or the pair ``(k, v)``,
     ``kv_of[i]`` the stacked key range the block of step ``i`` reads (of rank ``rank - i``:
     received by a ring, sliced from a held chunk by the single-GPU emulation), ``local_cu`` the
     device ``cu_seqlens`` of the own-chunk block of a packed chunk (batch 1).  ``before_rest`` is
@@ -240,7 +240,7 @@ def blocks_backward(q, kv, kv_of, out, lse, do, plan, scale, local_cu, dkv_of, k
         return _backward_two_blocks(q, kv[0], kv[1], kv_of[i1], dkv_of[i1], out, lse, do, plan,
                                     scale, local_cu, wide=True, after_rest=after_rest)
     dq = torch.empty(q.shape, dtype=torch.float32, device=q.device)
-    dkv = torch.empty(kv.shape, dtype=torch.float32, device=q.device)
+    dkv = torch.empty((2,) + tuple(kv[0].shape), dtype=torch.float32, device=q.device)
     first = True
     covered = q.shape[1]
     for (i, qs, _, window, causal) in plan[1:]:
@@ -269,7 +269,7 @@ def blocks_backward(q, kv, kv_of, out, lse, do, plan, scale, local_cu, dkv_of, k
 def _forward_blocks_accum(q, k, v, prev_kv, plan, scale, local_cu):
     """``blocks_forward`` on key ranges sliced from the held chunks of earlier ranks."""
     kv_of = {i: prev_kv[i - 1][:, :, ks] for (i, _, ks, _, _) in plan[1:]}
-    out, lse = blocks_forward(q, torch.stack([k, v]), kv_of, plan, scale, local_cu)
+    out, lse = blocks_forward(q, (k, v), kv_of, plan, scale, local_cu)
     return out.to(q.dtype), lse.float()
 
 
@@ -340,13 +340,13 @@ def _backward_blocks(q, k, v, prev_kv, out, lse, do, plan, scale, local_cu, ring
     if len(plan) == 1 and not ring_dtypes:
         # the own-chunk block alone (rank 0, or a window that ends inside the chunk for a pack
         # whose first sequence starts in it): 16-bit gradients straight from the kernels
-        dq, dkv = torch.empty_like(q), torch.empty_like(torch.stack([k, v]))
+        dq, dkv = torch.empty_like(q), torch.empty((2,) + tuple(k.shape), dtype=k.dtype, device=k.device)
         (_, _, _, window, causal) = plan[0]
         if local_cu is not None:
-            flash_attn_varlen_bwd_func(q, torch.stack([k, v]), out, lse, do, dq, dkv, local_cu,
+            flash_attn_varlen_bwd_func(q, (k, v), out, lse, do, dq, dkv, local_cu,
                                        local_cu, None, None, scale, window, causal)
         else:
-            flash_attn_bwd_func(q, torch.stack([k, v]), out, lse, do, dq, dkv, scale, window, causal)
+            flash_attn_bwd_func(q, (k, v), out, lse, do, dq, dkv, scale, window, causal)
         return (dq, dkv[0], dkv[1], *[torch.zeros_like(kv) for kv in prev_kv])
     if len(plan) == 2 and not ring_dtypes:
         one = _one_pass(q, k, v, prev_kv, plan, local_cu) if one_pass else None
@@ -365,7 +365,7 @@ def _backward_blocks(q, k, v, prev_kv, out, lse, do, plan, scale, local_cu, ring
     dprev = [torch.zeros_like(kv) for kv in prev_kv]
     kv_of = {i: prev_kv[i - 1][:, :, ks] for (i, _, ks, _, _) in plan[1:]}
     dkv_of = {i: dprev[i - 1][:, :, ks] for (i, _, ks, _, _) in plan[1:]}
-    dq, dkv = blocks_backward(q, torch.stack([k, v]), kv_of, out, lse, do, plan, scale, local_cu,
+    dq, dkv = blocks_backward(q, (k, v), kv_of, out, lse, do, plan, scale, local_cu,
                               dkv_of)
     return (dq.to(q.dtype), dkv[0].to(k.dtype), dkv[1].to(v.dtype), *dprev)
 
