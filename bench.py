@@ -31,7 +31,7 @@ PEAK_HBM_GBPS = 8000.0     # MI355X HBM3E
 # from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --pmc-pass`, each counter
 # scaled by what it reads for the 1 GiB device copy of that pass (FETCH_SIZE x2.0, WRITE_SIZE
 # x1.0); the summary is profiles/c3_step_kernels_hbm_traffic_pmc.txt.
-DKDV_HBM_BYTES_PER_LAUNCH = 748.2e6
+DKDV_HBM_BYTES_PER_LAUNCH = 757.4e6
 MERGE_HBM_BYTES_PER_LAUNCH = 5452.6e6
 # Untimed steps before the W warm-up steps: an idle GPU takes some tens of milliseconds of load to
 # settle its clocks (the first launches of a run take up to a third longer than the later ones), and
