@@ -154,6 +154,72 @@ def _mk(dev):
     return lambda *shape: torch.randn(*shape, device=dev, dtype=torch.bfloat16)
 
 
+def clock_probe(dev, qd, kd, vd, prev, do, S, W, seconds=4.0):
+    """Shader clock under each kernel of the step's band: every kernel is launched back to back
+    for ``seconds`` while a thread asks ``rocm-smi --showclocks`` five times a second; reported
+    are the median ``sclk`` of the readings taken after the first second and the kernel's launch
+    time over the same period.  The published matrix peak is priced at 2400 MHz."""
+    import re
+    import statistics
+    import subprocess
+    import threading
+    import time
+
+    import torch
+
+    from ring_swa.ops import attn_bwd, attn_fwd
+    from ring_swa.ops.band_attn import bwd_workspace_bytes
+
+    tk, tv = prev[0][:, S - W:], prev[1][:, S - W:]
+    dq, dk, dv = torch.empty_like(qd), torch.empty_like(kd), torch.empty_like(vd)
+    dtk, dtv = torch.empty_like(tk), torch.empty_like(tv)
+    big, big2 = (torch.empty(1 << 28, dtype=torch.float32, device=dev) for _ in range(2))
+    with torch.no_grad():
+        o_b, lse_b = attn_fwd(qd, tk, tv, None, (W, 0), True, second=(kd, vd))
+        ws = torch.empty(bwd_workspace_bytes(qd, tk, second_rows=S), dtype=torch.uint8, device=dev)
+        band = lambda ph: attn_bwd(qd, tk, tv, o_b, lse_b, do, dq, dtk, dtv, None, (W, 0), True,  # noqa: E731
+                                   workspace=ws, phases=ph, second=(kd, vd, dk, dv), handoff=False)
+        band(7)
+        kernels = [("attn_fwd_kernel", lambda: attn_fwd(qd, tk, tv, None, (W, 0), True, second=(kd, vd))),
+                   ("attn_bwd_dkdv_kernel", lambda: band(2)),
+                   ("attn_bwd_dq_kernel", lambda: band(4)),
+                   ("device copy of 1 GiB", lambda: big2.copy_(big))]
+        out = {}
+        for name, fn in kernels:
+            reads, stop = [], threading.Event()
+
+            def sample():
+                while not stop.is_set():
+                    try:
+                        txt = subprocess.run(["rocm-smi", "--showclocks", "--csv"], capture_output=True,
+                                             text=True, timeout=20).stdout
+                        m = re.search(r"\((\d+)Mhz\)[^()]*$", txt.strip().splitlines()[-1]) if txt.strip() else None
+                        if m:
+                            reads.append((time.time(), int(m.group(1))))
+                    except (OSError, subprocess.SubprocessError):
+                        pass
+                    time.sleep(0.2)
+
+            th = threading.Thread(target=sample)
+            th.start()
+            t0, times = time.time(), []
+            while time.time() - t0 < seconds:
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(50):
+                    fn()
+                e1.record()
+                torch.cuda.synchronize()
+                times.append(e0.elapsed_time(e1) / 50)
+            stop.set()
+            th.join()
+            late = [mhz for (t, mhz) in reads if t - t0 > 1.0]
+            out[name] = {"sclk_MHz_median": statistics.median(late) if late else None, "readings": len(late),
+                         "launch_ms_median": statistics.median(times[len(times) // 4:])}
+            time.sleep(1.0)
+    return {"clock_probe": out, "nominal_MHz": 2400}
+
+
 def case_c2(dev):
     """Configuration 2: plain single-GPU sliding-window attention, batch 2, seq 8192, 32 q = 32
     kv heads, head_dim 128, window 1000.  Returns (forward, backward, pairs x batch x heads)."""
@@ -259,6 +325,9 @@ def main():
     ap.add_argument("--pmc-pass", action="store_true",
                     help="counter-collection pass: launch a 1 GiB device copy (the known-size "
                          "calibration kernel) and every hot kernel twice, then exit")
+    ap.add_argument("--clock-probe", action="store_true",
+                    help="loop each kernel of the step's band for a few seconds and print the shader "
+                         "clock rocm-smi reads meanwhile (one JSON line; no timing claims)")
     ap.add_argument("--trace", choices=["c2", "c4", "c5"],
                     help="kernel-trace pass: run only that configuration's step a few times "
                          "(under rocprofv3 --kernel-trace --stats) and exit")
@@ -313,6 +382,10 @@ def main():
                 fn()
         torch.cuda.synchronize()
         print(json.dumps({"trace_pass": args.trace, "steps": args.steps}))
+        return
+
+    if args.clock_probe:
+        print(json.dumps(clock_probe(dev, q.detach(), k.detach(), v.detach(), prev.detach(), do, S, W)))
         return
 
     if args.pmc_pass:
